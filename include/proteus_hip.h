@@ -1,0 +1,157 @@
+/*
+ * proteus_hip.h -- C ABI of libproteus_hip.so (gfx950 / MI355X).
+ *
+ * Two operators of jaimec00/proteusAI behind plain pointers and sizes:
+ *   - the isotropic Wavefunction Embedding (WE) forward, and
+ *   - the RBF-scaled geometric flash-attention forward.
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers owned by the caller; the library borrows
+ *     them for the duration of the launch and keeps nothing.  Outputs are fully
+ *     overwritten (no reliance on zero-initialisation, no atomics).
+ *   - All tensors are dense and contiguous in the stated layout.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Launches are asynchronous; no entry point synchronises.
+ *   - Return value: 0 = launched; < 0 = argument error found BEFORE any HIP call
+ *     (so it can be exercised on a machine without a GPU); > 0 = a hipError_t
+ *     reported by the launch.  proteus_strerror() names any of them.
+ */
+#ifndef PROTEUS_HIP_H
+#define PROTEUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes (negative = argument errors) ---- */
+#define PROTEUS_OK                 0
+#define PROTEUS_ERR_NULL_POINTER  -1   /* a required pointer is NULL              */
+#define PROTEUS_ERR_BAD_SHAPE     -2   /* Z, N, K, H <= 0 or above the limits     */
+#define PROTEUS_ERR_BAD_HEAD_DIM  -3   /* d_head is not 64                        */
+#define PROTEUS_ERR_BAD_LAYOUT    -4   /* unknown coords_layout value             */
+#define PROTEUS_ERR_BAD_ALIGNMENT -5   /* a pointer is not aligned as required    */
+#define PROTEUS_ERR_BAD_TUNING    -6   /* unknown tuning/variant selector         */
+#define PROTEUS_ERR_UNSUPPORTED   -7   /* legacy option not implemented           */
+
+/* ---- coordinate layouts accepted by proteus_we_fwd ---- */
+#define PROTEUS_COORDS_SOA 0   /* [Z,3,N]: what the reference's wrapper hands its kernel */
+#define PROTEUS_COORDS_AOS 1   /* [Z,N,3]: what the Python module receives               */
+
+/* ---- limits ---- */
+#define PROTEUS_WE_MAX_N   (1 << 22)
+#define PROTEUS_WE_MAX_K   4096
+#define PROTEUS_ATTN_MAX_N (1 << 20)
+
+/* Library version (major*10000 + minor*100 + patch). */
+int proteus_version(void);
+
+/* Human-readable text for a return code of any entry point. */
+const char* proteus_strerror(int code);
+
+/*
+ * Isotropic Wavefunction Embedding forward (magnitude 1/|r|, no dropout).
+ *
+ * Replaces the reference's native entry `wf_embedding_kernel.forward(coords,
+ * wavenumbers, out, cos_sums, sin_sums, magnitude_type, dropout_p, rng_seed)`
+ *   utils/model_utils/wf_embedding/isotropic/cuda/wf_embedding_if.cpp:20-77
+ * and the launcher + kernel it calls
+ *   utils/model_utils/wf_embedding/isotropic/cuda/wf_embedding_kernel.cu:49-344
+ * for magnitude_type == 1 and dropout_p == 0 (the only values the module passes,
+ *   utils/model_utils/wf_embedding/wf_embedding.py:44).
+ *
+ * Semantics, for batch z, observer i, wavenumber k, with
+ *   valid(i,j) = !mask[z,i] && !mask[z,j] && |r_i - r_j|^2 != 0 :
+ *     out[z,i,2k]     = sum_j valid * cos(k_k r_ij) / r_ij
+ *     out[z,i,2k+1]   = sum_j valid * sin(k_k r_ij) / r_ij
+ *     cos_sums[z,i,k] = sum_j valid * cos(k_k r_ij)
+ *     sin_sums[z,i,k] = sum_j valid * sin(k_k r_ij)
+ *   A masked observer's rows are all zero.
+ *
+ * Difference from the reference: padding is an explicit byte mask (non-zero =
+ * padded) instead of the sentinel x == 12345 baked into the coordinates
+ * (isotropic/cuda/wf_embedding.py:29, wf_embedding_kernel.cu:154); a genuine
+ * coordinate of 12345.0 is therefore NOT masked here.
+ *
+ *   coords       [Z,3,N] or [Z,N,3] f32, per coords_layout
+ *   wavenumbers  [K] f32 (any sign)
+ *   mask         [Z,N] u8, non-zero = padded; may be NULL (nothing padded)
+ *   out          [Z,N,2K] f32     cos_sums, sin_sums  [Z,N,K] f32
+ *   tuning       0 = automatic; otherwise a variant selector (see
+ *                proteus_we_num_variants / proteus_we_variant_name)
+ */
+int proteus_we_fwd(const float* coords, int coords_layout,
+                   const float* wavenumbers, const uint8_t* mask,
+                   float* out, float* cos_sums, float* sin_sums,
+                   int Z, int N, int K, int tuning, void* stream);
+
+/* Validation half of proteus_we_fwd: same checks, no HIP call, no launch. */
+int proteus_we_fwd_check(const float* coords, int coords_layout,
+                         const float* wavenumbers, const uint8_t* mask,
+                         const float* out, const float* cos_sums, const float* sin_sums,
+                         int Z, int N, int K, int tuning);
+
+int         proteus_we_num_variants(void);
+const char* proteus_we_variant_name(int tuning);
+
+/*
+ * RBF-scaled geometric flash-attention forward.
+ *
+ * Replaces the Triton launch `_attn_fwd[grid](...)` made by
+ *   old/old_scripts/attn/geometric_attn.py:552-607 (kernel :57-260)
+ * with the logits of README.md:40:
+ *     s_ij = (q_i . k_j)/sqrt(d) * (1 + exp(-|r_i - r_j|^2 / (2 sigma_h^2)))
+ *     s_ij = -inf where key j is padded
+ *     O_i  = softmax_j(s_ij) V_j ;  L_i = logsumexp_j(s_ij)
+ *   Padded query rows and rows without any valid key give O = 0, L = -inf
+ *   (geometric_attn.py:196,233-236).
+ *
+ *   Q, K, V      [Z,H,N,64] bf16 (raw uint16 bit patterns), 16-byte aligned
+ *   coords       [Z,N,3] f32
+ *   sigma        [H] f32, > 0 (not checked on the device)
+ *   key_pad_mask [Z,N] u8, non-zero = padded; may be NULL
+ *   O            [Z,H,N,64] f32, 16-byte aligned
+ *   L            [Z,H,N] f32; may be NULL (then not written)
+ *   tuning       0 = automatic; otherwise a variant selector
+ */
+int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         const float* coords, const float* sigma,
+                         const uint8_t* key_pad_mask,
+                         float* O, float* L,
+                         int Z, int H, int N, int d_head, int tuning, void* stream);
+
+/* Validation half of proteus_geo_attn_fwd: same checks, no HIP call. */
+int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                               const float* coords, const float* sigma,
+                               const uint8_t* key_pad_mask,
+                               const float* O, const float* L,
+                               int Z, int H, int N, int d_head, int tuning);
+
+int         proteus_geo_attn_num_variants(void);
+const char* proteus_geo_attn_variant_name(int tuning);
+
+/*
+ * Instruction-rate probe used to state the roofline denominator of the WE
+ * kernel.  Runs `iters` rounds of 64 independent chains of one VALU
+ * instruction per lane on `blocks` x 256 threads and writes one float per
+ * thread to `sink` (so the work cannot be removed).  The caller times the
+ * launch; lane-ops issued = blocks*256*iters*64.  No counterpart in the
+ * reference.
+ *   op: 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_sin_f32, 4 v_cos_f32,
+ *       5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32
+ */
+int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
+
+/*
+ * Accuracy probe of the hardware sin/cos path used by the WE kernel:
+ * s[i] = v_sin_f32(fract(x[i])), c[i] = v_cos_f32(fract(x[i])) with x in
+ * revolutions, and q[i] = refined sqrt path r = r2*rsq(r2) applied to x[i].
+ */
+int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PROTEUS_HIP_H */

@@ -1,0 +1,89 @@
+"""ctypes front end of oracle/_build/liboracle.so (TEST INFRASTRUCTURE).
+
+The C sources cite the reference lines they follow; this file only marshals
+numpy arrays.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import build as _build
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = _build.LIB
+        if not os.path.exists(path):
+            _build.build()
+        _lib = ctypes.CDLL(path)
+    return _lib
+
+
+def _p(a, ct):
+    return None if a is None else a.ctypes.data_as(ctypes.POINTER(ct))
+
+
+def _rows(rows, N):
+    if rows is None:
+        return None, N
+    r = np.ascontiguousarray(np.asarray(rows, dtype=np.int32))
+    assert r.ndim == 1 and (r >= 0).all() and (r < N).all()
+    return r, int(r.shape[0])
+
+
+def we(coords, wavenumbers, mask=None, rows=None, precision="f64"):
+    """coords [Z,N,3], wavenumbers [K], mask [Z,N] bool (True = padded).
+
+    Returns (out [Z,R,2K], cos_sums [Z,R,K], sin_sums [Z,R,K]) for the selected
+    rows (all rows when rows is None), float64 for precision 'f64' and float32
+    for 'f32' (terms evaluated in float the way the PyTorch statement does).
+    """
+    c = np.ascontiguousarray(np.asarray(coords, dtype=np.float32))
+    w = np.ascontiguousarray(np.asarray(wavenumbers, dtype=np.float32))
+    Z, N, three = c.shape
+    assert three == 3
+    K = int(w.shape[0])
+    m = None if mask is None else np.ascontiguousarray(np.asarray(mask).astype(np.uint8))
+    if m is not None:
+        assert m.shape == (Z, N)
+    r, R = _rows(rows, N)
+    dt, ct, fn = (np.float64, ctypes.c_double, lib().we_oracle_f64) if precision == "f64" else \
+                 (np.float32, ctypes.c_float, lib().we_oracle_f32)
+    out = np.empty((Z, R, 2 * K), dt)
+    cs = np.empty((Z, R, K), dt)
+    ss = np.empty((Z, R, K), dt)
+    fn.restype = None
+    fn(_p(c, ctypes.c_float), _p(w, ctypes.c_float), _p(m, ctypes.c_uint8),
+       ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K), _p(r, ctypes.c_int), ctypes.c_int(R),
+       _p(out, ct), _p(cs, ct), _p(ss, ct))
+    return out, cs, ss
+
+
+def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, rows=None):
+    """Q,K,V [Z,H,N,d] (float values, already rounded to the kernel's operand
+    type by the caller), coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool.
+
+    Returns (O [Z,H,R,d], L [Z,H,R]) in float64.
+    """
+    q = np.ascontiguousarray(np.asarray(Q, dtype=np.float32))
+    k = np.ascontiguousarray(np.asarray(K, dtype=np.float32))
+    v = np.ascontiguousarray(np.asarray(V, dtype=np.float32))
+    c = np.ascontiguousarray(np.asarray(coords, dtype=np.float32))
+    s = np.ascontiguousarray(np.asarray(sigma, dtype=np.float32))
+    Z, H, N, d = q.shape
+    assert k.shape == q.shape and v.shape == q.shape and c.shape == (Z, N, 3) and s.shape == (H,)
+    m = None if key_padding_mask is None else np.ascontiguousarray(np.asarray(key_padding_mask).astype(np.uint8))
+    r, R = _rows(rows, N)
+    O = np.empty((Z, H, R, d), np.float64)
+    L = np.empty((Z, H, R), np.float64)
+    fn = lib().geo_attn_oracle_f64
+    fn.restype = None
+    fn(_p(q, ctypes.c_float), _p(k, ctypes.c_float), _p(v, ctypes.c_float), _p(c, ctypes.c_float),
+       _p(s, ctypes.c_float), _p(m, ctypes.c_uint8),
+       ctypes.c_int(Z), ctypes.c_int(H), ctypes.c_int(N), ctypes.c_int(d),
+       _p(r, ctypes.c_int), ctypes.c_int(R), _p(O, ctypes.c_double), _p(L, ctypes.c_double))
+    return O, L

@@ -1,0 +1,103 @@
+"""TEST INFRASTRUCTURE. The reference's CPU PyTorch path, restated and tiled.
+
+Not part of the product.  These are the functions whose time on the host
+cores is reported as the CPU baseline, and the fp32 checker of the parity
+tests.  Rows (observers / queries) are processed in chunks so temporaries stay
+bounded; rows are independent in both algorithms.
+"""
+import math
+
+import torch
+
+
+def we_torch(coords, wavenumbers, mask=None, rows=None, row_chunk=None, dtype=torch.float32,
+             max_temp_bytes=1 << 30):
+    """Isotropic wavefunction embedding, magnitude 1/|r|.
+
+    Follows tests/wf_embed/wf_embed.py:91-129 (wf_embedding_torch, mag_type 1):
+    dists = sqrt(sum((ci - cj)^2)); phases = dists*k; masked = mi | mj | dists==0;
+    magnitudes = 1/where(masked, inf, dists); real/imag = magnitudes*cos/sin(phases);
+    sum over sources; features = stack([real, imag], -1).view(Z, N, 2K).
+    The cos/sin sums follow isotropic/cuda/wf_embedding_kernel.cu:224-238
+    (warp_sum(real*dists)): sum over unmasked pairs of cos(phase), sin(phase).
+
+    coords [Z,N,3], wavenumbers [K], mask [Z,N] bool (True = padded).
+    Returns (out [Z,R,2K], cos_sums [Z,R,K], sin_sums [Z,R,K]).
+    """
+    coords = coords.to(dtype)
+    wavenumbers = wavenumbers.to(dtype)
+    Z, N, _ = coords.shape
+    K = wavenumbers.shape[0]
+    mask = torch.zeros(Z, N, dtype=torch.bool) if mask is None else mask.bool()
+    rows_t = torch.arange(N) if rows is None else torch.as_tensor(rows, dtype=torch.long)
+    R = rows_t.numel()
+    if row_chunk is None:
+        per_row = N * K * coords.element_size() * 4
+        row_chunk = max(1, min(R, max_temp_bytes // max(per_row, 1)))
+    out = torch.zeros(Z, R, 2 * K, dtype=dtype)
+    cs = torch.zeros(Z, R, K, dtype=dtype)
+    ss = torch.zeros(Z, R, K, dtype=dtype)
+    for z in range(Z):
+        cz, mz = coords[z], mask[z]
+        for a in range(0, R, row_chunk):
+            idx = rows_t[a:a + row_chunk]
+            ci = cz[idx]                                                     # r x 3
+            dists = torch.sqrt(torch.sum((ci[:, None, :] - cz[None, :, :]) ** 2, dim=2))   # r x N
+            phases = dists[:, :, None] * wavenumbers[None, None, :]          # r x N x K
+            m = mz[idx][:, None] | mz[None, :] | (dists == 0)                # r x N
+            mag = 1 / torch.where(m, torch.full_like(dists, float("inf")), dists)
+            valid = (~m).to(dtype)
+            cosp, sinp = torch.cos(phases), torch.sin(phases)
+            real = (mag[:, :, None] * cosp).sum(dim=1)
+            imag = (mag[:, :, None] * sinp).sum(dim=1)
+            out[z, a:a + idx.numel()] = torch.stack([real, imag], dim=-1).view(idx.numel(), 2 * K)
+            cs[z, a:a + idx.numel()] = (valid[:, :, None] * cosp).sum(dim=1)
+            ss[z, a:a + idx.numel()] = (valid[:, :, None] * sinp).sum(dim=1)
+    return out, cs, ss
+
+
+def we_backward_torch(dO, cos_sums, sin_sums):
+    """d(loss)/d(wavenumbers): isotropic/cuda/wf_embedding.py:64-83."""
+    real_dO = dO[:, :, 0::2]
+    imag_dO = dO[:, :, 1::2]
+    return ((imag_dO * cos_sums) - (real_dO * sin_sums)).sum(dim=(0, 1))
+
+
+def geo_attn_torch(Q, K, V, coords, sigma, key_padding_mask=None, rows=None, row_chunk=None,
+                   dtype=torch.float32, max_temp_bytes=1 << 30):
+    """RBF-scaled attention with the multiplier of README.md:40.
+
+    Dense structure of tests/attn/geo_attn.py:194-210 (S = QK^T/sqrt(d); dists;
+    rbfs = exp(-d^2/(2 sigma^2)); masked -> -inf; softmax; P V), with the logits
+    S*(1+rbf) and the conventions of old/old_scripts/attn/geometric_attn.py:
+    both padded queries and padded keys are masked (:196), a row without valid
+    keys gives O = 0 (:233) and L = -inf (:236).
+
+    Q,K,V [Z,H,N,d]; coords [Z,N,3]; sigma [H]; key_padding_mask [Z,N] bool.
+    Returns (O [Z,H,R,d], L [Z,H,R]).
+    """
+    Q, K, V = Q.to(dtype), K.to(dtype), V.to(dtype)
+    coords, sigma = coords.to(dtype), sigma.to(dtype)
+    Z, H, N, d = Q.shape
+    mask = torch.zeros(Z, N, dtype=torch.bool) if key_padding_mask is None else key_padding_mask.bool()
+    rows_t = torch.arange(N) if rows is None else torch.as_tensor(rows, dtype=torch.long)
+    R = rows_t.numel()
+    if row_chunk is None:
+        per_row = H * N * Q.element_size() * 4
+        row_chunk = max(1, min(R, max_temp_bytes // max(per_row, 1)))
+    O = torch.zeros(Z, H, R, d, dtype=dtype)
+    L = torch.full((Z, H, R), float("-inf"), dtype=dtype)
+    for z in range(Z):
+        for a in range(0, R, row_chunk):
+            idx = rows_t[a:a + row_chunk]
+            S = torch.matmul(Q[z][:, idx, :], K[z].transpose(1, 2)) / math.sqrt(d)      # H x r x N
+            d2 = torch.sum((coords[z][idx][:, None, :] - coords[z][None, :, :]) ** 2, dim=2)   # r x N
+            rbf = torch.exp(-d2[None] / (2 * sigma[:, None, None] ** 2))                # H x r x N
+            am = (mask[z][idx][:, None] | mask[z][None, :])[None]                       # 1 x r x N
+            S = torch.where(am, torch.full_like(S, float("-inf")), S * (1 + rbf))
+            Lz = torch.logsumexp(S, dim=-1)                                             # -inf for empty rows
+            P = torch.softmax(S, dim=-1)
+            P = torch.where(torch.isnan(P), torch.zeros_like(P), P)                     # empty rows -> 0
+            O[z][:, a:a + idx.numel()] = torch.matmul(P, V[z])
+            L[z][:, a:a + idx.numel()] = Lz
+    return O, L

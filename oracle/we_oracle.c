@@ -1,0 +1,103 @@
+/*
+ * TEST INFRASTRUCTURE -- CPU oracle of the isotropic Wavefunction Embedding.
+ * Not part of the product; the product path never links or calls this file.
+ *
+ * Follows, line by line in meaning:
+ *   tests/wf_embed/wf_embed.py:91-129                    (wf_embedding_torch, mag_type 1)
+ *   isotropic/cuda/wf_embedding_kernel.cu:181-250        (valid rule, sums = real*dists)
+ *   isotropic/triton_old/wf_embedding.py:163-198         (explicit-mask statement of the sums)
+ * under utils/model_utils/wf_embedding/.
+ *
+ *   dist_ij  = sqrt(sum_c (x_ic - x_jc)^2)                       wf_embed.py:100
+ *   phase    = dist_ij * k                                        wf_embed.py:103
+ *   masked   = mask_i | mask_j | dist_ij == 0                     wf_embed.py:106
+ *   mag      = 1 / (masked ? inf : dist_ij)                       wf_embed.py:112
+ *   out[i,2k]   = sum_j mag cos(phase), out[i,2k+1] = sum_j mag sin(phase)   wf_embed.py:119-127
+ *   cos_sums[i,k] = sum_j !masked cos(phase), sin_sums likewise   kernel.cu:224-238 (real*dists = cos)
+ *
+ * Two flavours: *_f64 evaluates everything in double; *_f32 evaluates each
+ * term in float exactly as the PyTorch statement would (sqrtf, float product,
+ * cosf/sinf, float divide) and accumulates the float terms in double.
+ * `rows` selects observers (NULL = all rows 0..nrows-1 of each batch item), so
+ * that long sequences can be checked on a sample: rows are independent.
+ * Output row r of batch z is written at index (z*nrows + r).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#define TILE_K 64
+
+void we_oracle_f64(const float* coords /*[Z,N,3]*/, const float* wn /*[K]*/,
+                   const uint8_t* mask /*[Z,N] or NULL*/, int Z, int N, int K,
+                   const int* rows, int nrows,
+                   double* out /*[Z,nrows,2K]*/, double* cs /*[Z,nrows,K]*/, double* ss)
+{
+    #pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int z = 0; z < Z; ++z)
+    for (int rr = 0; rr < nrows; ++rr) {
+        const int i = rows ? rows[rr] : rr;
+        const float* c = coords + (size_t)z * N * 3;
+        const uint8_t* m = mask ? mask + (size_t)z * N : NULL;
+        double* o = out + ((size_t)z * nrows + rr) * 2 * K;
+        double* pc = cs + ((size_t)z * nrows + rr) * K;
+        double* ps = ss + ((size_t)z * nrows + rr) * K;
+        for (int k = 0; k < K; ++k) { o[2*k] = o[2*k+1] = pc[k] = ps[k] = 0.0; }
+        if (m && m[i]) continue;
+        const double xi = c[3*i], yi = c[3*i+1], zi = c[3*i+2];
+        for (int j = 0; j < N; ++j) {
+            if (m && m[j]) continue;
+            const double dx = xi - c[3*j], dy = yi - c[3*j+1], dz = zi - c[3*j+2];
+            const double d2 = dx*dx + dy*dy + dz*dz;
+            if (d2 == 0.0) continue;
+            const double d = sqrt(d2), inv = 1.0 / d;
+            for (int k = 0; k < K; ++k) {
+                const double ph = d * (double)wn[k];
+                const double co = cos(ph), si = sin(ph);
+                o[2*k] += co * inv; o[2*k+1] += si * inv; pc[k] += co; ps[k] += si;
+            }
+        }
+    }
+}
+
+void we_oracle_f32(const float* coords, const float* wn, const uint8_t* mask, int Z, int N, int K,
+                   const int* rows, int nrows, float* out, float* cs, float* ss)
+{
+    #pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int z = 0; z < Z; ++z)
+    for (int rr = 0; rr < nrows; ++rr) {
+        const int i = rows ? rows[rr] : rr;
+        const float* c = coords + (size_t)z * N * 3;
+        const uint8_t* m = mask ? mask + (size_t)z * N : NULL;
+        float* o = out + ((size_t)z * nrows + rr) * 2 * K;
+        float* pc = cs + ((size_t)z * nrows + rr) * K;
+        float* ps = ss + ((size_t)z * nrows + rr) * K;
+        double* acc = (double*)calloc((size_t)4 * K, sizeof(double));
+        if (!(m && m[i])) {
+            const float xi = c[3*i], yi = c[3*i+1], zi = c[3*i+2];
+            for (int j = 0; j < N; ++j) {
+                if (m && m[j]) continue;
+                const float dx = xi - c[3*j], dy = yi - c[3*j+1], dz = zi - c[3*j+2];
+                /* torch: sum over the last dim of the squared differences, in float */
+                const float d2 = (dx*dx + dy*dy) + dz*dz;
+                const float d = sqrtf(d2);
+                if (d == 0.0f) continue;
+                const float inv = 1.0f / d;
+                for (int k = 0; k < K; ++k) {
+                    const float ph = d * wn[k];
+                    const float co = cosf(ph), si = sinf(ph);
+                    acc[4*k]   += (double)(inv * co);
+                    acc[4*k+1] += (double)(inv * si);
+                    acc[4*k+2] += (double)co;
+                    acc[4*k+3] += (double)si;
+                }
+            }
+        }
+        for (int k = 0; k < K; ++k) {
+            o[2*k] = (float)acc[4*k]; o[2*k+1] = (float)acc[4*k+1];
+            pc[k] = (float)acc[4*k+2]; ps[k] = (float)acc[4*k+3];
+        }
+        free(acc);
+    }
+}

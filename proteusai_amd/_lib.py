@@ -1,0 +1,85 @@
+"""ctypes binding of libproteus_hip.so (declarations in include/proteus_hip.h).
+
+There is no CPU fallback: if the library is missing or a call fails, an
+exception is raised.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libproteus_hip.so")
+
+COORDS_SOA = 0
+COORDS_AOS = 1
+
+# every symbol include/proteus_hip.h declares
+SYMBOLS = [
+    "proteus_version", "proteus_strerror",
+    "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_num_variants", "proteus_we_variant_name",
+    "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_num_variants",
+    "proteus_geo_attn_variant_name",
+    "proteus_probe_valu_rate", "proteus_probe_sincos",
+]
+
+_lib = None
+
+
+class ProteusError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the HIP library; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ProteusError(
+            f"{LIB_PATH} is missing: build it with `python -m proteusai_amd.build` "
+            "(there is no CPU fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.proteus_version.restype = ci
+    lib.proteus_strerror.restype = ctypes.c_char_p
+    lib.proteus_strerror.argtypes = [ci]
+    lib.proteus_we_fwd.restype = ci
+    lib.proteus_we_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.proteus_we_fwd_check.restype = ci
+    lib.proteus_we_fwd_check.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci]
+    lib.proteus_we_num_variants.restype = ci
+    lib.proteus_we_variant_name.restype = ctypes.c_char_p
+    lib.proteus_we_variant_name.argtypes = [ci]
+    lib.proteus_geo_attn_fwd.restype = ci
+    lib.proteus_geo_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.proteus_geo_attn_fwd_check.restype = ci
+    lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
+    lib.proteus_geo_attn_num_variants.restype = ci
+    lib.proteus_geo_attn_variant_name.restype = ctypes.c_char_p
+    lib.proteus_geo_attn_variant_name.argtypes = [ci]
+    lib.proteus_probe_valu_rate.restype = ci
+    lib.proteus_probe_valu_rate.argtypes = [ci, ci, ci, vp, vp]
+    lib.proteus_probe_sincos.restype = ci
+    lib.proteus_probe_sincos.argtypes = [vp, vp, vp, vp, ci, vp]
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str):
+    """Turn a return code into an exception: argument errors -> ValueError,
+    HIP errors -> ProteusError."""
+    if rc == 0:
+        return
+    msg = load().proteus_strerror(rc).decode()
+    if rc < 0:
+        raise ValueError(f"{what}: {msg} (code {rc})")
+    raise ProteusError(f"{what}: HIP error {rc}: {msg}")
+
+
+def we_variants():
+    lib = load()
+    return [lib.proteus_we_variant_name(i).decode() for i in range(lib.proteus_we_num_variants())]
+
+
+def geo_attn_variants():
+    lib = load()
+    return [lib.proteus_geo_attn_variant_name(i).decode() for i in range(lib.proteus_geo_attn_num_variants())]

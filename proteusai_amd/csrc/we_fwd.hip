@@ -1,0 +1,316 @@
+// Isotropic Wavefunction Embedding forward for gfx950 (MI355X).
+//
+// What it computes (reference semantics, magnitude 1/|r|, no dropout):
+//   utils/model_utils/wf_embedding/isotropic/cuda/wf_embedding_kernel.cu:181-250
+//   tests/wf_embed/wf_embed.py:91-129 (dense PyTorch statement)
+//
+// Mapping to the machine.  The reference gives one 64-thread block to one
+// observer, puts one source per thread and reduces every (source-block, k)
+// product across the warp with shuffles and shared-memory atomics.  Here the
+// roles are turned round so that no cross-lane traffic exists at all:
+//   - a LANE owns one observer i; a WAVE owns 64 observers and a tile of KT
+//     wavenumbers, whose 4*KT running sums live in VGPRs for the whole kernel;
+//   - the wavenumbers of the tile are wave-uniform and sit in SGPRs;
+//   - sources are streamed: the workgroup (4 waves = the same 64 observers,
+//     4 wavenumber tiles) stages blocks of source coordinates in LDS, already
+//     compacted to the unpadded ones, and every lane reads the same source with
+//     one broadcast ds_read_b128;
+//   - per (pair, k) the wave issues: v_mul (phase, in revolutions), v_fract,
+//     v_sin, v_cos, 2 x v_fmac (embedding), 2 x v_add (cos/sin sums).
+// Padded sources never reach the inner loop (compaction), padded observers are
+// computed as ordinary lanes and written as zeros, and the self/coincident pair
+// (r^2 == 0) runs through the loop with r = 0 and 1/r = 0: it adds exactly
+// cos(0) = 1 to each cos sum and nothing else, and the count of such pairs is
+// subtracted once at the end.  No branch in the inner loop depends on a lane.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "proteus_hip.h"
+
+namespace {
+
+constexpr int WE_WAVES   = 4;
+constexpr int WE_THREADS = WE_WAVES * 64;
+constexpr int WE_JB      = 256;   // sources staged per LDS block (one per thread)
+
+__device__ __forceinline__ float sgpr(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
+// KT     wavenumbers per wave (4*KT accumulators per lane)
+// SPLIT  the sources are split over gridDim.x/ceil(N/64) workgroups and partial
+//        sums are added to pre-zeroed outputs with float atomics (small N only)
+template <int KT, bool SPLIT>
+__global__ __launch_bounds__(WE_THREADS)
+void we_fwd_kernel(const float* __restrict__ coords, const int layout,
+                   const float* __restrict__ wavenumbers,
+                   const uint8_t* __restrict__ mask,
+                   float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
+                   const int N, const int K, const int nsplit)
+{
+    __shared__ float4 s_keys[WE_JB + 1];   // +1: the stream loop reads one source ahead
+    __shared__ int    s_wcount[WE_WAVES];
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int z    = blockIdx.z;
+
+    int iblock = blockIdx.x, split = 0;
+    if (SPLIT) { iblock = blockIdx.x / nsplit; split = blockIdx.x - iblock * nsplit; }
+
+    const size_t zN = (size_t)z * (size_t)N;
+    const float* cz = coords + zN * 3;
+    const uint8_t* mz = mask ? mask + zN : nullptr;
+
+    // ---- this lane's observer ----
+    const int  i      = iblock * 64 + lane;
+    const bool i_in   = i < N;
+    const int  ic     = i_in ? i : N - 1;
+    float xi, yi, zi;
+    if (layout == PROTEUS_COORDS_SOA) { xi = cz[ic]; yi = cz[(size_t)N + ic]; zi = cz[2 * (size_t)N + ic]; }
+    else                              { xi = cz[3 * (size_t)ic]; yi = cz[3 * (size_t)ic + 1]; zi = cz[3 * (size_t)ic + 2]; }
+    const bool i_valid = i_in && !(mz && mz[ic]);
+
+    // Every wave of the workgroup sees the same 64 observers, so this exit is
+    // uniform over the workgroup and happens before the first barrier.
+    const bool any_valid = __builtin_amdgcn_ballot_w64(i_valid) != 0;
+
+    // ---- this wave's wavenumbers, converted to revolutions per angstrom ----
+    const int  k0          = (blockIdx.y * WE_WAVES + wave) * KT;
+    const bool wave_active = k0 < K;
+    float kr[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        const int k = k0 + t;
+        const float w = (k < K) ? wavenumbers[k] : 0.0f;
+        kr[t] = sgpr((float)((double)w * 0.15915494309189533577));
+    }
+
+    float acc_oc[KT], acc_os[KT], acc_c[KT], acc_s[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) { acc_oc[t] = 0.f; acc_os[t] = 0.f; acc_c[t] = 0.f; acc_s[t] = 0.f; }
+    float nzero = 0.f;
+
+    if (any_valid) {
+        // sources handled by this workgroup
+        int j_begin = 0, j_end = N;
+        if (SPLIT) {
+            const int chunk = ((N + nsplit - 1) / nsplit + WE_JB - 1) / WE_JB * WE_JB;
+            j_begin = split * chunk;
+            j_end   = min(N, j_begin + chunk);
+        }
+
+        for (int jb = j_begin; jb < j_end; jb += WE_JB) {
+            // -- stage one block of sources, keeping only the unpadded ones --
+            const int  j    = jb + tid;
+            const bool j_in = j < j_end;
+            const int  jc   = j_in ? j : N - 1;
+            float xj, yj, zj;
+            if (layout == PROTEUS_COORDS_SOA) { xj = cz[jc]; yj = cz[(size_t)N + jc]; zj = cz[2 * (size_t)N + jc]; }
+            else                              { xj = cz[3 * (size_t)jc]; yj = cz[3 * (size_t)jc + 1]; zj = cz[3 * (size_t)jc + 2]; }
+            const bool j_valid = j_in && !(mz && mz[jc]);
+
+            const uint64_t bal   = __builtin_amdgcn_ballot_w64(j_valid);
+            const int      below = __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+            __syncthreads();                       // previous block fully consumed
+            if (lane == 0) s_wcount[wave] = __builtin_popcountll(bal);
+            __syncthreads();
+            int base = 0, nk = 0;
+#pragma unroll
+            for (int w = 0; w < WE_WAVES; ++w) { const int c = s_wcount[w]; base += (w < wave) ? c : 0; nk += c; }
+            if (j_valid) s_keys[base + below] = make_float4(xj, yj, zj, 0.f);
+            __syncthreads();
+            nk = __builtin_amdgcn_readfirstlane(nk);
+
+            if (!wave_active) continue;
+
+            // -- stream the staged sources --
+            float4 knext = s_keys[0];
+#pragma unroll 1
+            for (int jj = 0; jj < nk; ++jj) {
+                const float4 kj = knext;
+                knext = s_keys[jj + 1];
+                const float dx = xi - kj.x, dy = yi - kj.y, dz = zi - kj.z;
+                const float r2 = dx * dx + dy * dy + dz * dz;
+                const bool  ok = r2 != 0.0f;
+                const float inv = ok ? __builtin_amdgcn_rsqf(r2) : 0.0f;
+                // one Newton step on r = r2 * rsq(r2): r is then within 1 ulp of sqrt(r2)
+                const float r0 = r2 * inv;
+                const float e  = __builtin_fmaf(-r0, r0, r2);
+                const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
+                nzero += ok ? 0.0f : 1.0f;
+#pragma unroll
+                for (int t = 0; t < KT; ++t) {
+                    const float ph = __builtin_amdgcn_fractf(r * kr[t]);
+                    const float s  = __builtin_amdgcn_sinf(ph);
+                    const float c  = __builtin_amdgcn_cosf(ph);
+                    acc_oc[t] = __builtin_fmaf(c, inv, acc_oc[t]);
+                    acc_os[t] = __builtin_fmaf(s, inv, acc_os[t]);
+                    acc_c[t] += c;
+                    acc_s[t] += s;
+                }
+            }
+        }
+    }
+
+    if (!wave_active || !i_in) return;
+
+    // ---- epilogue: each lane writes its own rows ----
+    const size_t row = zN + (size_t)i;
+    float* o  = out      + row * (size_t)(2 * K) + 2 * (size_t)k0;
+    float* pc = cos_sums + row * (size_t)K + k0;
+    float* ps = sin_sums + row * (size_t)K + k0;
+
+    if (SPLIT) {
+        if (!i_valid) return;                    // outputs were pre-zeroed
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            if (k0 + t < K) {
+                unsafeAtomicAdd(o + 2 * t,     acc_oc[t]);
+                unsafeAtomicAdd(o + 2 * t + 1, acc_os[t]);
+                unsafeAtomicAdd(pc + t, acc_c[t] - nzero);
+                unsafeAtomicAdd(ps + t, acc_s[t]);
+            }
+        }
+        return;
+    }
+
+    const float keep = i_valid ? 1.0f : 0.0f;    // padded observer: zeros
+    if (k0 + KT <= K && (K & 1) == 0 && (KT & 3) == 0 && (K & 3) == 0) {
+        // full tile, rows 16-byte aligned: vector stores
+#pragma unroll
+        for (int t = 0; t < KT; t += 2) {
+            float4 v = make_float4(acc_oc[t] * keep, acc_os[t] * keep, acc_oc[t + 1] * keep, acc_os[t + 1] * keep);
+            *reinterpret_cast<float4*>(o + 2 * t) = v;
+        }
+#pragma unroll
+        for (int t = 0; t < KT; t += 4) {
+            float4 c = make_float4((acc_c[t] - nzero) * keep, (acc_c[t + 1] - nzero) * keep,
+                                   (acc_c[t + 2] - nzero) * keep, (acc_c[t + 3] - nzero) * keep);
+            float4 s = make_float4(acc_s[t] * keep, acc_s[t + 1] * keep, acc_s[t + 2] * keep, acc_s[t + 3] * keep);
+            *reinterpret_cast<float4*>(pc + t) = c;
+            *reinterpret_cast<float4*>(ps + t) = s;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            if (k0 + t < K) {
+                o[2 * t]     = acc_oc[t] * keep;
+                o[2 * t + 1] = acc_os[t] * keep;
+                pc[t] = (acc_c[t] - nzero) * keep;
+                ps[t] = acc_s[t] * keep;
+            }
+        }
+    }
+}
+
+__global__ void we_zero_kernel(float4* p, size_t n4, float* tail, int ntail) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n4; idx += stride)
+        p[idx] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (blockIdx.x == 0 && (int)threadIdx.x < ntail) tail[threadIdx.x] = 0.f;
+}
+
+void zero_async(float* p, size_t n, hipStream_t st) {
+    // a plain fill kernel rather than a memset node, so callers may capture it
+    const size_t n4 = n / 4;
+    const int ntail = (int)(n - n4 * 4);
+    const int blocks = (int)((n4 + 255) / 256 > 4096 ? 4096 : ((n4 + 255) / 256 ? (n4 + 255) / 256 : 1));
+    hipLaunchKernelGGL(we_zero_kernel, dim3(blocks), dim3(256), 0, st,
+                       reinterpret_cast<float4*>(p), n4, p + n4 * 4, ntail);
+}
+
+struct WeVariant { const char* name; int kt; bool split; };
+// index 0 is "automatic"; the others force a tile
+const WeVariant kVariants[] = {
+    {"auto", 0, false},
+    {"kt32", 32, false},
+    {"kt16", 16, false},
+    {"kt8", 8, false},
+    {"kt64", 64, false},
+    {"kt32_split", 32, true},
+    {"kt16_split", 16, true},
+    {"kt8_split", 8, true},
+};
+constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
+
+template <int KT, bool SPLIT>
+int launch(const float* coords, int layout, const float* wn, const uint8_t* mask,
+           float* out, float* cs, float* ss, int Z, int N, int K, int nsplit, hipStream_t st)
+{
+    const int iblocks = (N + 63) / 64;
+    const int ktiles  = (K + KT * WE_WAVES - 1) / (KT * WE_WAVES);
+    if (SPLIT) {
+        zero_async(out, (size_t)Z * N * 2 * K, st);
+        zero_async(cs,  (size_t)Z * N * K, st);
+        zero_async(ss,  (size_t)Z * N * K, st);
+    }
+    dim3 grid(iblocks * (SPLIT ? nsplit : 1), ktiles, Z);
+    hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT>), grid, dim3(WE_THREADS), 0, st,
+                       coords, layout, wn, mask, out, cs, ss, N, K, nsplit);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" int proteus_we_num_variants(void) { return kNumVariants; }
+
+extern "C" const char* proteus_we_variant_name(int tuning) {
+    return (tuning >= 0 && tuning < kNumVariants) ? kVariants[tuning].name : nullptr;
+}
+
+extern "C" int proteus_we_fwd_check(const float* coords, int coords_layout,
+                                    const float* wavenumbers, const uint8_t* mask,
+                                    const float* out, const float* cos_sums, const float* sin_sums,
+                                    int Z, int N, int K, int tuning)
+{
+    (void)mask;
+    if (!coords || !wavenumbers || !out || !cos_sums || !sin_sums) return PROTEUS_ERR_NULL_POINTER;
+    if (Z <= 0 || N <= 0 || K <= 0) return PROTEUS_ERR_BAD_SHAPE;
+    if (N > PROTEUS_WE_MAX_N || K > PROTEUS_WE_MAX_K || Z > 65535) return PROTEUS_ERR_BAD_SHAPE;
+    if (coords_layout != PROTEUS_COORDS_SOA && coords_layout != PROTEUS_COORDS_AOS) return PROTEUS_ERR_BAD_LAYOUT;
+    if (tuning < 0 || tuning >= kNumVariants) return PROTEUS_ERR_BAD_TUNING;
+    if (((uintptr_t)out & 15) || ((uintptr_t)cos_sums & 15) || ((uintptr_t)sin_sums & 15)) return PROTEUS_ERR_BAD_ALIGNMENT;
+    return PROTEUS_OK;
+}
+
+extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
+                              const float* wavenumbers, const uint8_t* mask,
+                              float* out, float* cos_sums, float* sin_sums,
+                              int Z, int N, int K, int tuning, void* stream)
+{
+    const int rc = proteus_we_fwd_check(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+
+    int kt = kVariants[tuning].kt;
+    bool split = kVariants[tuning].split;
+    const long iblocks = ((long)N + 63) / 64 * Z;
+    if (tuning == 0) {
+        // Aim for at least two waves on each of the 1024 SIMDs; prefer the
+        // widest wavenumber tile (least per-pair overhead) that achieves it.
+        const long want = 2048;
+        kt = 32;
+        while (kt > 8 && iblocks * ((K + kt - 1) / kt) < want) kt >>= 1;
+        if (kt > K) { kt = 8; while (kt < K && kt < 32) kt <<= 1; }
+        split = iblocks * ((K + kt - 1) / kt) < want / 2 && N >= 2 * WE_JB;
+    }
+    int nsplit = 1;
+    if (split) {
+        const long waves = iblocks * ((K + kt - 1) / kt);
+        nsplit = (int)((2048 + waves - 1) / waves);
+        const int maxsplit = (N + WE_JB - 1) / WE_JB;
+        if (nsplit > maxsplit) nsplit = maxsplit;
+        if (nsplit < 1) nsplit = 1;
+    }
+#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, nsplit, st) \
+                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, st))
+    switch (kt) {
+        case 64: return launch<64, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, st);
+        case 32: return WE_GO(32);
+        case 16: return WE_GO(16);
+        default: return WE_GO(8);
+    }
+#undef WE_GO
+}

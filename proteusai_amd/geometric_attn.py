@@ -1,0 +1,136 @@
+"""RBF-scaled geometric attention operator and module on the HIP kernel.
+
+Mirrors the reference's Python surface:
+  geometric_attn(...) / _geometric_attn   old/old_scripts/attn/geometric_attn.py:545-607
+  GeoAttention                            old/old_scripts/encoder.py:43-121
+with the logits of README.md:40, s = (q.k/sqrt(d)) * (1 + exp(-|rq-rk|^2/(2 sigma_h^2))),
+plus `geo_attn`, the (Q, K, V, coords, sigma_per_head, key_padding_mask) form.
+"""
+import torch
+import torch.nn as nn
+
+from . import _lib
+
+
+def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0):
+    """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None).
+
+    Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569),
+    coords and sigma to fp32; O is fp32 [Z,H,N,d] as in the reference (:578).
+    key_padding_mask: True = padded.  Padded query rows and rows without a
+    valid key give O = 0 and logsumexp = -inf.  With return_lse the
+    logsumexp L [Z,H,N] is returned as well.
+    """
+    if not (Q.shape == K.shape == V.shape):
+        raise AssertionError(f"Q, K, and V projection shapes must match, but got {Q.shape=}, {K.shape=}, {V.shape=}")
+    if Q.dim() != 4:
+        raise AssertionError(f"Q, K, V must be of shape (batch, heads, N, d_k), not {tuple(Q.shape)}")
+    Z, H, N, d = Q.shape
+    if coords.dim() != 3 or coords.size(2) != 3 or coords.size(0) != Z or coords.size(1) != N:
+        raise AssertionError(f"coordinates must be of shape (batch, N, 3), not {tuple(coords.shape)}")
+    if sigma.dim() != 1 or sigma.size(0) != H:
+        raise AssertionError(f"number of spreads must be equal to nheads, not {tuple(sigma.shape)} and {H=}")
+    if not Q.is_cuda:
+        raise _lib.ProteusError("geo_attn needs tensors on the GPU (there is no CPU path)")
+    if not bool(torch.all(sigma > 0)):
+        raise AssertionError(f"spreads must be a tensor of positive, non-zero floats, not {sigma}")
+    lib = _lib.load()
+    dev = Q.device
+    q = Q.detach().to(torch.bfloat16).contiguous()
+    k = K.detach().to(torch.bfloat16).contiguous()
+    v = V.detach().to(torch.bfloat16).contiguous()
+    c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
+    s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
+    m = None
+    if key_padding_mask is not None:
+        if tuple(key_padding_mask.shape) != (Z, N):
+            raise AssertionError(f"mask must be of shape ({Z}, {N}), not {tuple(key_padding_mask.shape)}")
+        m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
+    O = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
+    L = torch.empty(Z, H, N, dtype=torch.float32, device=dev)
+    if Z == 0 or H == 0 or N == 0:
+        return (O, L) if return_lse else O
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
+                                      None if m is None else m.data_ptr(),
+                                      O.data_ptr(), L.data_ptr(), Z, H, N, d, int(tuning), stream)
+    _lib.check(rc, "proteus_geo_attn_fwd")
+    return (O, L) if return_lse else O
+
+
+class _geometric_attn(torch.autograd.Function):
+    """Forward only: the backward kernel of the reference (geometric_attn.py:262-543) is not implemented."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, coords, spreads, key_padding_mask):
+        return geo_attn(Q, K, V, coords, spreads, key_padding_mask)
+
+    @staticmethod
+    def backward(ctx, dO):
+        raise NotImplementedError("geometric attention backward is not implemented")
+
+
+def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00):
+    """Same call as the reference's geometric_attn (geometric_attn.py:545-548).
+
+    The logits are the README form S*(1+RBF); the reference kernel's
+    beta-weighted bias S + beta*RBF_norm*|S| and its [min_rbf, max_rbf] pair
+    mask are not implemented: `betas` must be None and the rbf range must be
+    the full [0, 1].
+    """
+    if betas is not None:
+        raise NotImplementedError("the beta-weighted bias of the legacy kernel is not implemented; pass betas=None")
+    if min_rbf > 0.0 or max_rbf < 1.0:
+        raise NotImplementedError("the [min_rbf, max_rbf] pair mask is not implemented; use min_rbf=0, max_rbf=1")
+    return _geometric_attn.apply(Q, K, V, coords, spreads, mask)
+
+
+class GeoAttention(nn.Module):
+    """Multi-head attention whose logits are scaled per head by 1 + RBF of the
+    pairwise C-alpha distance.  Constructor, parameters and forward follow
+    old/old_scripts/encoder.py:43-121 (per-head QKV projections with bias,
+    sigma = min_spread + exp(w), heads concatenated as a (d_k x heads)
+    interleave, bias-free output projection).  beta_weights is kept so that
+    state dicts line up, but does not enter the logits."""
+
+    def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=0.0, max_rbf=1.00, learn_spreads=True):
+        super().__init__()
+        self.heads = heads
+        self.d_model = d_model
+        if self.d_model % self.heads != 0:
+            raise ValueError(f"number of dimensions ({self.d_model}) must be divisible by number of attention heads ({self.heads})")
+        self.d_k = self.d_model // self.heads
+        self.spread_weights = nn.Parameter(torch.zeros(heads), requires_grad=learn_spreads)
+        self.beta_weights = nn.Parameter(torch.zeros(heads))
+        self.min_spread = min_spread
+        self.min_rbf = min_rbf
+        self.max_rbf = max_rbf
+        xavier_scale = (6 / (self.d_k + d_model)) ** 0.5
+        self.q_proj = nn.Parameter(-xavier_scale + torch.rand(self.heads, self.d_model, self.d_k) * (2 * xavier_scale))
+        self.k_proj = nn.Parameter(-xavier_scale + torch.rand(self.heads, self.d_model, self.d_k) * (2 * xavier_scale))
+        self.v_proj = nn.Parameter(-xavier_scale + torch.rand(self.heads, self.d_model, self.d_k) * (2 * xavier_scale))
+        self.q_bias = nn.Parameter(torch.zeros(self.heads, self.d_k))
+        self.k_bias = nn.Parameter(torch.zeros(self.heads, self.d_k))
+        self.v_bias = nn.Parameter(torch.zeros(self.heads, self.d_k))
+        self.out_proj = nn.Linear(d_model, d_model, bias=False)
+
+    def get_spreads(self):
+        return self.min_spread + torch.exp(self.spread_weights)
+
+    def get_betas(self):
+        return torch.exp(self.beta_weights)
+
+    def forward(self, q, k, v, coords, mask=None):
+        assert q.shape == k.shape == v.shape
+        assert q.dim() == 3
+        batch, N, d_model = q.shape
+        assert d_model == self.d_model
+        Q = torch.matmul(q.unsqueeze(1), self.q_proj.unsqueeze(0)) + self.q_bias.unsqueeze(0).unsqueeze(2)
+        K = torch.matmul(k.unsqueeze(1), self.k_proj.unsqueeze(0)) + self.k_bias.unsqueeze(0).unsqueeze(2)
+        V = torch.matmul(v.unsqueeze(1), self.v_proj.unsqueeze(0)) + self.v_bias.unsqueeze(0).unsqueeze(2)
+        out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, min_rbf=self.min_rbf, max_rbf=self.max_rbf)
+        out = out.to(q.dtype)
+        out = out.permute(0, 2, 3, 1)                    # batch x N x d_k x heads
+        out = out.reshape(batch, N, self.d_model)
+        return self.out_proj(out)

@@ -1,0 +1,111 @@
+"""Wavefunction Embedding operator and module on the HIP kernel.
+
+Mirrors the reference's Python surface for the isotropic path:
+  wf_embedding(...) / _wf_embedding      utils/model_utils/wf_embedding/isotropic/cuda/wf_embedding.py:18-83
+  WaveFunctionEmbedding                  utils/model_utils/wf_embedding/wf_embedding.py:24-46
+plus `we_forward`, which also returns the per-token cos/sin sums.
+"""
+import torch
+import torch.nn as nn
+
+from . import _lib
+
+
+def we_forward(coords, wavenumbers, mask=None, tuning: int = 0):
+    """out, cos_sums, sin_sums = we_forward(coords [Z,N,3], wavenumbers [K], mask [Z,N] bool | None).
+
+    mask: True = padded.  Unlike the reference wrapper (which crashes on
+    mask=None at isotropic/cuda/wf_embedding.py:29), None means "nothing padded".
+    All outputs are float32 on coords' device: out [Z,N,2K] with cos terms at
+    even and sin terms at odd feature indices, cos_sums / sin_sums [Z,N,K].
+    """
+    if coords.dim() != 3 or coords.size(2) != 3:
+        raise ValueError(f"coords must be of shape (batch, N, 3), not {tuple(coords.shape)}")
+    if wavenumbers.dim() != 1:
+        raise ValueError(f"wavenumbers must be of shape (K,), not {tuple(wavenumbers.shape)}")
+    if not coords.is_cuda:
+        raise _lib.ProteusError("we_forward needs tensors on the GPU (there is no CPU path)")
+    lib = _lib.load()
+    dev = coords.device
+    # everything in fp32, as isotropic/cuda/wf_embedding.py:32-35
+    c = coords.detach().to(torch.float32).contiguous()
+    w = wavenumbers.detach().to(device=dev, dtype=torch.float32).contiguous()
+    Z, N, _ = c.shape
+    K = w.shape[0]
+    m = None
+    if mask is not None:
+        if tuple(mask.shape) != (Z, N):
+            raise ValueError(f"mask must be of shape ({Z}, {N}), not {tuple(mask.shape)}")
+        m = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
+    out = torch.empty(Z, N, 2 * K, dtype=torch.float32, device=dev)
+    cos_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev)
+    sin_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev)
+    if Z == 0 or N == 0 or K == 0:
+        return out, cos_sums, sin_sums
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
+                                None if m is None else m.data_ptr(),
+                                out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
+                                Z, N, K, int(tuning), stream)
+    _lib.check(rc, "proteus_we_fwd")
+    return out, cos_sums, sin_sums
+
+
+class _wf_embedding(torch.autograd.Function):
+    """Forward on the HIP kernel; analytical O(N K) backward for the wavenumbers
+    (isotropic/cuda/wf_embedding.py:64-83).  No gradient flows to coords, as in
+    the reference."""
+
+    @staticmethod
+    def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask):
+        if magnitude_type not in (0, 1, 2, 3):
+            raise AssertionError("magnitude_type must be one of 0, 1, 2, 3")
+        if magnitude_type != 1:
+            raise NotImplementedError("only magnitude_type=1 (1/|R|) is implemented; it is the only value "
+                                      "the WaveFunctionEmbedding module passes")
+        if dropout_p != 0.0:
+            raise NotImplementedError("dropout_p != 0 is not implemented; the module always passes 0.0")
+        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask)
+        ctx.save_for_backward(cos_sums, sin_sums)
+        ctx.wn_dtype = wavenumbers.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dO):
+        cos_sums, sin_sums = ctx.saved_tensors
+        real_dO = dO[:, :, 0::2]
+        imag_dO = dO[:, :, 1::2]
+        dk = ((imag_dO * cos_sums) - (real_dO * sin_sums)).sum(dim=(0, 1))
+        return None, dk.to(ctx.wn_dtype), None, None, None
+
+
+def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None):
+    """Same call as the reference's wf_embedding (isotropic/cuda/wf_embedding.py:18)."""
+    return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask)
+
+
+class WaveFunctionEmbedding(nn.Module):
+    """Same constructor and forward as utils/model_utils/wf_embedding/wf_embedding.py:24-46.
+
+    The wavelength schedule follows the code (torch.logspace, endpoint
+    inclusive), the parameter holds log(wavenumber).  Only the isotropic branch
+    exists here; anisotropic=True (the reference default) raises.
+    """
+
+    def __init__(self, d_wf=512, min_wl=4.0, max_wl=35.0, base_wl=20.0, anisotropic=True, learn_wl=False, learn_aa=False):
+        super().__init__()
+        wl = min_wl + (max_wl - min_wl) * ((torch.logspace(0, 1, d_wf // 2, base_wl) - 1) / (base_wl - 1))
+        wn = torch.log(torch.pi * 2 / wl)
+        self.wavenumbers = nn.Parameter(wn, requires_grad=learn_wl)
+        self.aa_magnitudes = nn.Parameter(torch.ones(d_wf // 2), requires_grad=learn_aa)
+        self.aniso = anisotropic
+
+    def get_wavenumbers(self):
+        return torch.exp(self.wavenumbers)
+
+    def forward(self, coords_alpha, coords_beta=None, key_padding_mask=None):
+        if self.aniso:
+            raise NotImplementedError("the anisotropic (C-beta scaled) embedding is not implemented; "
+                                      "construct with anisotropic=False")
+        return wf_embedding(coords_alpha, self.get_wavenumbers(), magnitude_type=1, dropout_p=0.0, mask=key_padding_mask)
