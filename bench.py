@@ -1,0 +1,207 @@
+"""Headline benchmark: Wavefunction Embedding forward at B=1, N=16384, d_model=512
+(BASELINE.json configs[1]) on one MI355X, with the geometric attention forward at
+N=16384, H=8, d=64 measured beside it, roofline fractions for both kernels and
+the CPU PyTorch path timed on the host cores as a baseline.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-attn]
+
+Prints ONE JSON line.  A "step" is one WE forward over the whole batch, inputs
+and outputs resident in HBM, outputs pre-allocated.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks used as roofline denominators
+PEAK_FP32_VECTOR_TFLOPS = 157.3     # packed-FMA vector fp32
+PEAK_BF16_MFMA_TFLOPS = 2500.0      # dense bf16 matrix
+H100_REFERENCE_GPW = 6.87194767e10 / 0.386 / 1e9   # README.md:34: 386 ms at this exact shape on an H100
+
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), bytes
+WE_TRAFFIC_BYTES = None
+ATTN_TRAFFIC_BYTES = None
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def probe_rates(lib, torch, dev):
+    """Measured lane-op rates (lane-ops/s) of the instructions the WE inner loop issues."""
+    names = ["fma", "mul", "add", "sin", "cos", "exp2", "rsq", "fract"]
+    sink = torch.empty(2048 * 256, device=dev)
+    rates = {}
+    for op, name in enumerate(names):
+        blocks, iters = 2048, 1000
+        lib.proteus_probe_valu_rate(op, blocks, iters, sink.data_ptr(), None)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        lib.proteus_probe_valu_rate(op, blocks, iters, sink.data_ptr(), None)
+        e1.record()
+        torch.cuda.synchronize()
+        rates[name] = blocks * 256 * iters * 64 / (e0.elapsed_time(e1) * 1e-3)
+    return rates
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-attn", action="store_true", help="skip the geometric attention leg")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--we-tuning", type=int, default=0)
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also launch a 256 MiB device copy, so a rocprofv3 --pmc run of this command holds a kernel of known traffic")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially, see DESIGN.md); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from proteusai_amd import _lib, synth
+    lib = _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------- WE forward, B=1, N=16384, d_model=512, compacted random-walk chain ----------------
+    Z, N, d_model = 1, 16384, 512
+    coords, wn = synth.we_inputs(N, seed=2, batch=Z, d_model=d_model, compact=True)
+    K = wn.numel()
+    c, w = coords.to(dev).contiguous(), wn.to(dev)
+    out = torch.empty(Z, N, 2 * K, device=dev)
+    cs = torch.empty(Z, N, K, device=dev)
+    ss = torch.empty(Z, N, K, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def we_step():
+        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(), None, out.data_ptr(), cs.data_ptr(),
+                                ss.data_ptr(), Z, N, K, args.we_tuning, stream)
+        if rc != 0:
+            _lib.check(rc, "proteus_we_fwd")
+
+    for _ in range(args.warmup):
+        we_step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e0, e1 in evs:
+        e0.record()
+        we_step()
+        e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
+    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+    ms_per_step = elapsed * 1e3 / args.steps
+    W = float(Z) * N * N * K                          # pair*wavenumber evaluations per step
+    value = W * args.steps / elapsed / 1e9            # Gpair*wavenumber/s, whole job
+
+    rates = probe_rates(lib, torch, dev)
+    r_valu = (rates["fma"] + rates["mul"] + rates["add"]) / 3
+    r_trans = (rates["sin"] + rates["cos"]) / 2
+    t_model_ms = W * (5.0 / r_valu + 2.0 / r_trans) * 1e3       # 5 fp32 VALU + 2 transcendental lane-ops per unit
+    achieved_tflops = 9.0 * W / (avg_kernel_ms * 1e-3) / 1e12   # 9 flop per unit, FMA counted as 2
+    roofline = {
+        "kernel": "we_fwd_kernel", "bound": "valu", "achieved": achieved_tflops, "peak": PEAK_FP32_VECTOR_TFLOPS,
+        "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_FP32_VECTOR_TFLOPS, "traffic": WE_TRAFFIC_BYTES,
+        "kernel_ms": avg_kernel_ms,
+        "issue_model": {
+            "lane_ops_per_unit": {"valu_fp32": 5, "transcendental": 2},
+            "measured_rate_valu_lane_ops_per_s": r_valu, "measured_rate_trans_lane_ops_per_s": r_trans,
+            "model_ms": t_model_ms, "frac": t_model_ms / avg_kernel_ms,
+        },
+    }
+
+    result = {
+        "metric": "we_fwd_gpair_wavenumber_per_s", "value": value, "unit": "Gpair*wavenumber/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": value / H100_REFERENCE_GPW,
+        "baseline_note": "reference README.md:34: 386 ms (178 Gpair*wavenumber/s) for this shape on an H100",
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "WE forward B=1 N=16384 d_model=512 (256 wavenumbers), compacted random-walk C-alpha chain, "
+                               "lambda 3.7-20 A base 20, no mask (BASELINE.json configs[1])",
+                   "Z": Z, "N": N, "K": K, "we_variant": _lib.we_variants()[args.we_tuning]},
+        "roofline": roofline,
+    }
+
+    # ---------------- geometric attention forward, N=16384, H=8, d=64 (configs[4]) ----------------
+    if not args.no_attn:
+        wc, _ = synth.we_inputs(65536, seed=5, compact=True)
+        Q, Kt, V, ac, sigma, _ = synth.attn_inputs(1, 8, 16384, 64, seed=5, coords=wc[:, :16384].contiguous())
+        q, k, v, acd, sg = Q.to(dev), Kt.to(dev), V.to(dev), ac.to(dev), sigma.to(dev)
+        O = torch.empty(1, 8, 16384, 64, device=dev)
+        L = torch.empty(1, 8, 16384, device=dev)
+
+        def attn_step():
+            rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), acd.data_ptr(), sg.data_ptr(), None,
+                                          O.data_ptr(), L.data_ptr(), 1, 8, 16384, 64, 0, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_geo_attn_fwd")
+        for _ in range(max(3, args.warmup)):
+            attn_step()
+        torch.cuda.synchronize()
+        n_it = max(10, args.steps)
+        aev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_it)]
+        for e0, e1 in aev:
+            e0.record()
+            attn_step()
+            e1.record()
+        torch.cuda.synchronize()
+        a_ms = sum(e0.elapsed_time(e1) for e0, e1 in aev) / n_it
+        flops = 4.0 * 8 * 64 * 16384 * 16384
+        a_tflops = flops / (a_ms * 1e-3) / 1e12
+        result["geo_attn"] = {
+            "workload": "geometric attention forward Z=1 H=8 N=16384 d_head=64 bf16, compacted chain, sigma 3-25 A (BASELINE.json configs[4])",
+            "ms": a_ms, "tflops": a_tflops, "dtype": "bf16",
+            "roofline": {"kernel": "geo_attn_fwd_kernel", "bound": "mfma", "achieved": a_tflops, "peak": PEAK_BF16_MFMA_TFLOPS,
+                         "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES},
+        }
+
+    # ---------------- CPU baseline: the tiled CPU PyTorch path on a bounded sample of observer rows ----------------
+    if not args.no_cpu:
+        from oracle import torch_oracle
+        threads = torch.get_num_threads()
+        rows = 64
+        t = time.perf_counter()
+        torch_oracle.we_torch(coords, wn, rows=list(range(rows)))
+        dt = time.perf_counter() - t
+        rows = int(max(64, min(N, rows * args.cpu_seconds / max(dt, 1e-3))))
+        rows -= rows % 64
+        sel = torch.linspace(0, N - 1, rows).long().tolist()
+        t = time.perf_counter()
+        torch_oracle.we_torch(coords, wn, rows=sel)
+        dt = time.perf_counter() - t
+        result["cpu_baseline"] = {
+            "value": rows * float(N) * K / dt / 1e9, "unit": "Gpair*wavenumber/s", "cores": threads, "kind": "port",
+            "sample": f"{rows} of {N} observer rows of the same workload (all {N} sources each), tiled CPU PyTorch fp32, {dt:.1f} s",
+            "host_cpus": os.cpu_count(),
+        }
+
+    if args.copy_calib:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

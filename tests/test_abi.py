@@ -1,0 +1,168 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every
+symbol the header declares, validates arguments before touching HIP, and the
+Python operator layer mirrors the reference's surface and error behaviour."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import proteusai_amd as pa
+from proteusai_amd import _lib, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "proteus_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(proteus_[a-z0-9_]+)\s*\(", header)))
+    assert declared, "no declarations found in the header"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in proteus_hip.h but not exported"
+    assert sorted(declared) == sorted(_lib.SYMBOLS)
+
+
+def test_version_and_strerror():
+    lib = _lib.load()
+    assert lib.proteus_version() >= 100
+    assert lib.proteus_strerror(0) == b"ok"
+    for code in range(-7, 0):
+        assert lib.proteus_strerror(code) not in (b"", b"unknown error code")
+    assert lib.proteus_strerror(-99) == b"unknown error code"
+
+
+def test_we_argument_validation_happens_before_any_hip_call():
+    lib = _lib.load()
+    p = 0x1000  # an aligned, never dereferenced address
+    ok = dict(coords=p, layout=0, wn=p, mask=None, out=p, cs=p, ss=p, Z=1, N=8, K=4, tuning=0)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return lib.proteus_we_fwd_check(a["coords"], a["layout"], a["wn"], a["mask"], a["out"], a["cs"], a["ss"],
+                                        a["Z"], a["N"], a["K"], a["tuning"])
+    assert call() == 0
+    for name in ("coords", "wn", "out", "cs", "ss"):
+        assert call(**{name: None}) == -1
+    for name in ("Z", "N", "K"):
+        assert call(**{name: 0}) == -2 and call(**{name: -3}) == -2
+    assert call(N=(1 << 22) + 1) == -2 and call(K=4097) == -2
+    assert call(layout=2) == -4
+    assert call(out=p + 4) == -5
+    assert call(tuning=999) == -6 and call(tuning=-1) == -6
+    # the launching entry point runs the same checks first: a bad argument never reaches the GPU
+    assert lib.proteus_we_fwd(None, 0, p, None, p, p, p, 1, 8, 4, 0, None) == -1
+    assert lib.proteus_we_fwd(p, 7, p, None, p, p, p, 1, 8, 4, 0, None) == -4
+
+
+def test_attention_argument_validation():
+    lib = _lib.load()
+    p = 0x1000
+    ok = [p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0]
+
+    def call(idx=None, val=None):
+        a = list(ok)
+        if idx is not None:
+            a[idx] = val
+        return lib.proteus_geo_attn_fwd_check(*a)
+    assert call() == 0
+    for idx in (0, 1, 2, 3, 4, 6):
+        assert call(idx, None) == -1
+    assert call(7, None) == 0                  # L is optional
+    for idx in (8, 9, 10):
+        assert call(idx, 0) == -2
+    assert call(11, 32) == -3 and call(11, 128) == -3
+    assert call(12, 55) == -6
+    assert call(0, p + 2) == -5
+    assert lib.proteus_geo_attn_fwd(p, p, p, p, p, None, p, p, 1, 2, 16, 48, 0, None) == -3
+
+
+def test_check_raises_python_exceptions():
+    with pytest.raises(ValueError):
+        _lib.check(-2, "x")
+    with pytest.raises(_lib.ProteusError):
+        _lib.check(700, "x")
+    _lib.check(0, "x")
+
+
+def test_variant_tables():
+    assert _lib.we_variants()[0] == "auto" and len(_lib.we_variants()) == _lib.load().proteus_we_num_variants()
+    assert _lib.geo_attn_variants()[0] == "auto"
+    assert _lib.load().proteus_we_variant_name(10 ** 6) is None
+
+
+def test_operators_refuse_cpu_tensors_instead_of_falling_back():
+    coords = torch.randn(1, 8, 3)
+    with pytest.raises(_lib.ProteusError):
+        pa.we_forward(coords, torch.rand(4))
+    with pytest.raises(_lib.ProteusError):
+        pa.wf_embedding(coords, torch.rand(4), mask=torch.zeros(1, 8, dtype=torch.bool))
+    Q = torch.randn(1, 2, 8, 64)
+    with pytest.raises(_lib.ProteusError):
+        pa.geo_attn(Q, Q, Q, coords, torch.ones(2))
+
+
+def test_operator_argument_errors_match_the_reference_surface():
+    coords = torch.randn(1, 8, 3)
+    with pytest.raises(ValueError):
+        pa.we_forward(torch.randn(1, 8, 2), torch.rand(4))
+    with pytest.raises(AssertionError):
+        pa.wf_embedding(coords, torch.rand(4), magnitude_type=5)
+    with pytest.raises(NotImplementedError):
+        pa.wf_embedding(coords, torch.rand(4), magnitude_type=0)
+    with pytest.raises(NotImplementedError):
+        pa.wf_embedding(coords, torch.rand(4), dropout_p=0.1)
+    Q = torch.randn(1, 2, 8, 64)
+    with pytest.raises(AssertionError):
+        pa.geo_attn(Q, Q[:, :, :4], Q, coords, torch.ones(2))
+    with pytest.raises(AssertionError):
+        pa.geo_attn(Q, Q, Q, coords[:, :, :2], torch.ones(2))
+    with pytest.raises(AssertionError):
+        pa.geo_attn(Q, Q, Q, coords, torch.ones(3))
+    with pytest.raises(NotImplementedError):
+        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), betas=torch.ones(2))
+    with pytest.raises(NotImplementedError):
+        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), None, min_rbf=0.1)
+
+
+def test_wavefunction_embedding_module_schedule_and_parameters():
+    # utils/model_utils/wf_embedding/wf_embedding.py:30-37: logspace(0,1,K,base) is endpoint inclusive
+    m = pa.WaveFunctionEmbedding(d_wf=512, min_wl=3.7, max_wl=20.0, base_wl=20.0, anisotropic=False, learn_wl=True)
+    wl = 2 * torch.pi / m.get_wavenumbers()
+    assert wl.shape == (256,)
+    assert wl[0].item() == pytest.approx(3.7, rel=1e-5) and wl[-1].item() == pytest.approx(20.0, rel=1e-5)
+    assert torch.all(wl[1:] > wl[:-1])
+    assert m.wavenumbers.requires_grad and not m.aa_magnitudes.requires_grad
+    assert set(dict(m.named_parameters())) == {"wavenumbers", "aa_magnitudes"}
+    with pytest.raises(NotImplementedError):
+        pa.WaveFunctionEmbedding()(torch.randn(1, 4, 3), torch.randn(1, 4, 3))
+
+
+def test_geo_attention_module_parameters():
+    m = pa.GeoAttention(d_model=512, heads=8, min_spread=2.0)
+    names = set(dict(m.named_parameters()))
+    assert names == {"spread_weights", "beta_weights", "q_proj", "k_proj", "v_proj", "q_bias", "k_bias", "v_bias", "out_proj.weight"}
+    assert tuple(m.q_proj.shape) == (8, 512, 64)
+    assert torch.allclose(m.get_spreads(), torch.full((8,), 3.0))
+    with pytest.raises(ValueError):
+        pa.GeoAttention(d_model=100, heads=8)
+
+
+def test_synthetic_inputs():
+    g = torch.Generator().manual_seed(0)
+    x = synth.random_walk_chain(500, g)
+    bonds = (x[1:] - x[:-1]).double().norm(dim=1)
+    assert torch.allclose(bonds, torch.full_like(bonds, 3.8), atol=1e-3)
+    y = synth.compact_chain(x, g)
+    assert synth.radius_of_gyration(y) == pytest.approx(2.2 * 500 ** 0.38, rel=1e-4)
+    wl = synth.wavelength_schedule(512)
+    assert wl[0].item() == pytest.approx(3.7) and wl[-1].item() < 20.0 and wl.shape == (256,)
+    s = synth.log_spaced_sigma(8)
+    assert s[0].item() == pytest.approx(3.0) and s[-1].item() == pytest.approx(25.0)
+    c1, w1 = synth.we_inputs(64, 5)
+    c2, w2 = synth.we_inputs(64, 5)
+    assert torch.equal(c1, c2) and torch.equal(w1, w2)
+    Q, K, V, c, sg, m = synth.attn_inputs(2, 2, 100, 64, 3, min_len=50)
+    assert Q.dtype == torch.bfloat16 and m.shape == (2, 100) and (~m).sum(1).min() >= 50

@@ -1,0 +1,212 @@
+"""GPU parity tests of the RBF-scaled geometric attention forward: the HIP
+kernel, called through the C ABI, against the CPU oracles evaluated on the
+bf16-rounded operands.
+
+Bar: max |O - O_ref| <= 2e-2 (bf16 operands, fp32 accumulation) on rows the
+reference defines; padded / empty rows must be exactly 0 with L = -inf."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import proteusai_amd as pa
+from oracle import c_oracle
+from proteusai_amd import _lib, synth
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS_TOL = 2e-2         # the stated parity bar for bf16 attention
+LSE_TOL = 1e-3             # the logsumexp never sees bf16 probabilities
+
+
+def make(seed, Z, H, N, qscale=1.0, maskfrac=0.0, tail=False):
+    g = torch.Generator().manual_seed(seed)
+    Q = (torch.randn(Z, H, N, 64, generator=g) * qscale).bfloat16()
+    K = (torch.randn(Z, H, N, 64, generator=g) * qscale).bfloat16()
+    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    coords = torch.stack([synth.random_walk_chain(N, g) for _ in range(Z)])
+    sigma = synth.log_spaced_sigma(H)
+    mask = None
+    if maskfrac > 0:
+        mask = torch.rand(Z, N, generator=g) < maskfrac
+    if tail:
+        lens = torch.randint(max(1, N // 2), N + 1, (Z,), generator=g)
+        t = torch.arange(N)[None, :] >= lens[:, None]
+        mask = t if mask is None else (mask | t)
+    return Q, K, V, coords, sigma, mask
+
+
+def run_gpu(gpu, Q, K, V, coords, sigma, mask):
+    O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu),
+                       None if mask is None else mask.to(gpu), return_lse=True)
+    torch.cuda.synchronize()
+    return O.cpu().numpy(), L.cpu().numpy()
+
+
+def check(got, Q, K, V, coords, sigma, mask, rows=None, what=""):
+    O, L = got
+    Or, Lr = c_oracle.geo_attn(Q.float().numpy(), K.float().numpy(), V.float().numpy(), coords.numpy(), sigma.numpy(),
+                               None if mask is None else mask.numpy(), rows=rows)
+    sel = slice(None) if rows is None else np.asarray(rows)
+    O, L = O[:, :, sel].astype(np.float64), L[:, :, sel].astype(np.float64)
+    assert np.isfinite(O).all(), f"{what}: non-finite output"
+    err = np.abs(O - Or).max()
+    assert err <= MAX_ABS_TOL, f"{what}: max abs error {err:.3e}"
+    fin = np.isfinite(Lr)
+    assert (np.isneginf(L) == ~fin).all(), f"{what}: -inf pattern of L differs"
+    if fin.any():
+        assert np.abs(L[fin] - Lr[fin]).max() <= LSE_TOL, f"{what}: logsumexp error {np.abs(L[fin] - Lr[fin]).max():.3e}"
+    assert (O[~fin] == 0).all(), f"{what}: padded / empty rows must be exactly zero"
+    return err
+
+
+@pytest.mark.parametrize("N", [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 513])
+def test_ragged_lengths(gpu, N):
+    a = make(100 + N, 2, 3, N)
+    check(run_gpu(gpu, *a), *a, what=f"N={N}")
+
+
+def test_golden_fixture(gpu, golden_dir):
+    g = np.load(os.path.join(golden_dir, "geo_attn_small.npz"))
+    t = [torch.from_numpy(g[k]) for k in ("Q", "K", "V", "coords", "sigma", "mask")]
+    O, L = run_gpu(gpu, t[0].bfloat16(), t[1].bfloat16(), t[2].bfloat16(), t[3], t[4], t[5])
+    assert np.abs(O - g["O"]).max() <= MAX_ABS_TOL
+    fin = np.isfinite(g["L"])
+    assert (np.isneginf(L) == ~fin).all() and np.abs(L[fin] - g["L"][fin]).max() <= LSE_TOL
+    assert (O[~fin] == 0).all()
+
+
+def test_masks(gpu):
+    N = 300
+    Q, K, V, coords, sigma, _ = make(1, 5, 2, N)
+    g = torch.Generator().manual_seed(1)
+    mask = torch.zeros(5, N, dtype=torch.bool)
+    mask[0] = torch.rand(N, generator=g) < 0.5       # scattered
+    mask[1, 131:] = True                             # tail padding, not tile aligned
+    mask[2] = True                                   # everything padded
+    mask[3] = True
+    mask[3, 77] = False                              # one valid token
+    mask[4, :64] = True                              # a whole leading key tile padded
+    check(run_gpu(gpu, Q, K, V, coords, sigma, mask), Q, K, V, coords, sigma, mask, what="masks")
+
+
+def test_large_logits(gpu):
+    # logits of order +-40: the online softmax must not overflow or lose the maximum
+    a = make(2, 1, 4, 400, qscale=2.5)
+    check(run_gpu(gpu, *a), *a, what="large logits")
+
+
+def test_flat_multiplier_equals_sdpa_on_gpu(gpu):
+    # sigma -> infinity: multiplier == 2 -> torch SDPA with scale 2/sqrt(d), evaluated in fp32 on the same bf16 values
+    Q, K, V, coords, _, _ = make(3, 2, 4, 777)
+    sigma = torch.full((4,), 1e7)
+    O, _ = run_gpu(gpu, Q, K, V, coords, sigma, None)
+    ref = F.scaled_dot_product_attention(Q.float().to(gpu), K.float().to(gpu), V.float().to(gpu), scale=2 / 8).cpu().numpy()
+    assert np.abs(O - ref).max() <= MAX_ABS_TOL
+
+
+def test_softmax_rows_sum_to_one(gpu):
+    Q, K, V, coords, sigma, mask = make(4, 2, 8, 1000, tail=True)
+    O, L = run_gpu(gpu, Q, K, torch.ones_like(V), coords, sigma, mask)
+    valid = ~mask.numpy()
+    for z in range(2):
+        assert np.abs(O[z][:, valid[z]] - 1).max() < 1e-2 and (O[z][:, ~valid[z]] == 0).all()
+
+
+def test_key_padding_equals_truncation(gpu):
+    Q, K, V, coords, sigma, _ = make(5, 1, 2, 260)
+    mask = torch.zeros(1, 260, dtype=torch.bool)
+    mask[0, 200:] = True
+    O, L = run_gpu(gpu, Q, K, V, coords, sigma, mask)
+    O2, L2 = run_gpu(gpu, Q[:, :, :200].contiguous(), K[:, :, :200].contiguous(), V[:, :, :200].contiguous(),
+                     coords[:, :200].contiguous(), sigma, None)
+    assert np.array_equal(O[:, :, :200], O2) and np.array_equal(L[:, :, :200], L2)
+
+
+def test_rigid_motion_of_coordinates(gpu):
+    Q, K, V, coords, sigma, _ = make(6, 1, 4, 500)
+    O, _ = run_gpu(gpu, Q, K, V, coords, sigma, None)
+    g = torch.Generator().manual_seed(6)
+    q, _ = torch.linalg.qr(torch.randn(3, 3, generator=g, dtype=torch.float64))
+    moved = (coords.double() @ q.T + torch.tensor([10.0, -20.0, 5.0], dtype=torch.float64)).float()
+    O2, _ = run_gpu(gpu, Q, K, V, moved, sigma, None)
+    assert np.abs(O - O2).max() < 5e-3
+
+
+def test_raw_c_abi_without_lse_and_canaries(gpu):
+    Q, K, V, coords, sigma, _ = make(7, 1, 2, 150)
+    lib = _lib.load()
+    n, pad = 1 * 2 * 150 * 64, 64
+    buf = torch.full((n + 2 * pad,), -777.0, device=gpu)
+    buf[pad:pad + n] = float("nan")
+    q, k, v, c, s = Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu)
+    rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(), None,
+                                  buf.data_ptr() + 4 * pad, None, 1, 2, 150, 64, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    h = buf.cpu()
+    assert (h[:pad] == -777.0).all() and (h[pad + n:] == -777.0).all()
+    O = h[pad:pad + n].view(1, 2, 150, 64).numpy()
+    Or, _ = c_oracle.geo_attn(Q.float().numpy(), K.float().numpy(), V.float().numpy(), coords.numpy(), sigma.numpy())
+    assert np.abs(O - Or).max() <= MAX_ABS_TOL
+
+
+def test_deterministic(gpu):
+    a = make(8, 2, 4, 900, tail=True)
+    x, y = run_gpu(gpu, *a), run_gpu(gpu, *a)
+    assert np.array_equal(x[0], y[0]) and np.array_equal(x[1], y[1])
+
+
+def test_module_forward_matches_composition(gpu):
+    # GeoAttention: per-head projections -> op -> (d_k x heads) interleaved concat -> out_proj
+    torch.manual_seed(0)
+    mod = pa.GeoAttention(d_model=128, heads=2, min_spread=2.0).to(gpu)
+    with torch.no_grad():
+        mod.spread_weights.copy_(torch.tensor([0.3, 1.2]))
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(2, 90, 128, generator=g)
+    coords = torch.stack([synth.random_walk_chain(90, g) for _ in range(2)])
+    mask = torch.zeros(2, 90, dtype=torch.bool)
+    mask[1, 60:] = True
+    with torch.no_grad():
+        y = mod(x.to(gpu), x.to(gpu), x.to(gpu), coords.to(gpu), mask=mask.to(gpu)).cpu()
+        p = {k: v.detach().cpu() for k, v in mod.named_parameters()}
+        Qh = torch.matmul(x.unsqueeze(1), p["q_proj"].unsqueeze(0)) + p["q_bias"][None, :, None]
+        Kh = torch.matmul(x.unsqueeze(1), p["k_proj"].unsqueeze(0)) + p["k_bias"][None, :, None]
+        Vh = torch.matmul(x.unsqueeze(1), p["v_proj"].unsqueeze(0)) + p["v_bias"][None, :, None]
+        sig = 2.0 + torch.exp(p["spread_weights"])
+        Or, _ = c_oracle.geo_attn(Qh.bfloat16().float().numpy(), Kh.bfloat16().float().numpy(), Vh.bfloat16().float().numpy(),
+                                  coords.numpy(), sig.numpy(), mask.numpy())
+        ref = torch.from_numpy(Or).float().permute(0, 2, 3, 1).reshape(2, 90, 128) @ p["out_proj.weight"].T
+    assert (y - ref).abs().max() < 5e-2
+
+
+def test_cfg3_sampled_rows(gpu):
+    # B=4, N=4096, H=8, d=64, Q,K,V ~ N(0,1)/8, lengths in [2048, 4096]
+    Q, K, V, coords, sigma, mask = synth.attn_inputs(4, 8, 4096, 64, seed=3, min_len=2048)
+    got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
+    rows = np.sort(np.random.default_rng(3).choice(4096, 64, replace=False)).astype(np.int32)
+    check(got, Q, K, V, coords, sigma, mask, rows=rows, what="cfg3")
+
+
+def test_cfg3_shape_with_unit_variance_logits(gpu):
+    # same shape, but logits of order one so that the softmax is far from uniform
+    Q, K, V, coords, sigma, mask = make(33, 4, 8, 4096, tail=True)
+    got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
+    rows = np.sort(np.random.default_rng(33).choice(4096, 48, replace=False)).astype(np.int32)
+    check(got, Q, K, V, coords, sigma, mask, rows=rows, what="cfg3 unit-variance")
+
+
+def test_cfg5_sampled_rows(gpu):
+    # N=16384, H=8, d=64 on the first 16384 residues of the compacted N=65536 chain
+    wc, _ = synth.we_inputs(65536, seed=5, compact=True)
+    Q, K, V, coords, sigma, mask = synth.attn_inputs(1, 8, 16384, 64, seed=5, coords=wc[:, :16384].contiguous())
+    got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
+    rows = np.sort(np.random.default_rng(5).choice(16384, 32, replace=False)).astype(np.int32)
+    check(got, Q, K, V, coords, sigma, mask, rows=rows, what="cfg5")
+    # size-independent property at full size: V = 1 -> O = 1
+    O1, _ = run_gpu(gpu, Q, K, torch.ones_like(V), coords, sigma, None)
+    assert np.abs(O1 - 1).max() < 1e-2
