@@ -18,6 +18,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 instructions are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results stay in ordinary VGPRs: the softmax reads every accumulator element on
+    # the vector ALU, and AGPR-resident accumulators would cost a v_accvgpr_read/write per access
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-command-line-argument",
     "-I", INCLUDE,
 ]

@@ -7,20 +7,34 @@
 //
 // Mapping to the machine.  A workgroup is 4 waves; a wave owns 32 queries of one
 // (batch, head) and walks the keys in tiles of 64 that the workgroup stages in
-// LDS (K row-major, V transposed, key coordinates pre-scaled for the head).
-// Both products run on v_mfma_f32_32x32x16_bf16 and are computed TRANSPOSED:
+// LDS (K row-major, V transposed, key geometry).  All products run on the matrix
+// cores and are computed TRANSPOSED:
 //   S^T (keys x queries)  = K_tile (A, from LDS) x Q^T (B, registers, loaded once)
+//   D^T (keys x queries)  = G_tile (A, from LDS) x G_q^T (B, registers)     [geometry, see below]
 //   O^T (d x queries)    += V^T_tile (A, from LDS) x P^T (B, registers)
 // In the 32x32 accumulator layout a lane holds 16 rows of ONE column, so with
 // queries on the columns each lane owns one query: the row maximum, the
 // exponentials and the row sum are in-lane except for one exchange between the
 // two half-waves, and the S^T accumulator registers are, after conversion to
-// bf16, already the B operand of the second product (the contraction index is
+// bf16, already the B operand of the last product (the contraction index is
 // merely visited in the permuted order the accumulator layout dictates, and the
 // V^T operand is read from LDS in that same order).
-// The geometric multiplier is evaluated per score from the lane's query
-// coordinates and broadcast reads of the staged key coordinates; nothing of
-// size N x N exists anywhere.
+//
+// Geometry on the matrix cores.  With x' = (x - c) * sqrt(log2(e)/2)/sigma_h (c = a
+// point near the workgroup's queries) the multiplier is 1 + exp2(D),
+//   D = -|x'_k - x'_q|^2 = -|x'_k|^2 + 2 x'_k . x'_q - |x'_q|^2 .
+// Every fp32 scalar is split exactly into three bf16 pieces (8+8+8 mantissa
+// bits), and D becomes a 24-term bf16 contraction whose products are exact in
+// the fp32 accumulator: per coordinate the pieces hh, hm, mh, mm, hl, lh (the
+// dropped ml, lm, ll are below 2^-24 of the product), plus the two squared
+// norms against ones.  One 32x32x16 and one 32x32x8 MFMA per 32 keys replace six
+// vector-ALU instructions per score.  The cancellation error is about
+// 2^-20 (|x'_k|^2 + |x'_q|^2); it only matters where the multiplier differs from
+// 1, i.e. for keys within ~6 sigma of the query, so with the origin near the
+// queries it is below 3e-3 in D as long as the workgroup's queries lie within
+// GA_MFMA_DIST_MAX_RHO2 of that origin.  A workgroup whose queries are spread
+// wider evaluates the distances directly on the vector ALU instead.
+// Nothing of size N x N exists anywhere.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -29,10 +43,10 @@
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float  floatx16 __attribute__((ext_vector_type(16)));
 typedef float  floatx2 __attribute__((ext_vector_type(2)));
+typedef short  shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int GA_WAVES   = 4;
 constexpr int GA_THREADS = GA_WAVES * 64;
@@ -41,15 +55,27 @@ constexpr int GA_BN      = 64;              // keys per tile
 constexpr int GA_D       = 64;              // head dim
 constexpr int GA_LDK     = GA_D + 8;        // LDS row stride of the K tile (bf16 elements)
 constexpr int GA_LDV     = GA_BN + 8;       // LDS row stride of the V^T tile
+constexpr int GA_LDG     = 40;              // LDS row stride of the key geometry tile (24 used)
 constexpr float LOG2E    = 1.4426950408889634f;
+// Largest squared distance (scaled units) of a workgroup's queries from their origin for
+// which the matrix-core distance path is used.
+constexpr float GA_MFMA_DIST_MAX_RHO2 = 1000.0f;
 
-struct __align__(16) Smem {
+// One staged key tile.  Two of them are kept so that the next tile can be written
+// while the current one is still being read (one barrier per tile).
+struct __align__(16) TileBuf {
     uint16_t k[GA_BN * GA_LDK];      // K tile   [key][d]
     uint16_t vt[GA_D * GA_LDV];      // V^T tile [d][key]
-    float    cx[GA_BN], cy[GA_BN], cz[GA_BN];   // key coordinates * sqrt(log2(e)/(2 sigma^2))
+    uint16_t geo[GA_BN * GA_LDG];    // key side of the distance contraction, 24 bf16 per key
+    float    cx[GA_BN], cy[GA_BN], cz[GA_BN];   // scaled key coordinates (vector-ALU distance path)
     float    bias[GA_BN];            // 0 for a valid key, -inf for a padded / out-of-range one
-    int      flags[2];               // [0] tile has a masked key, [1] tile has a valid key
+    int      flags[4];               // [0] tile has a masked key, [1] tile has a valid key
+};
+
+struct __align__(16) Smem {
+    TileBuf  tile[2];
     int      n_eff;                  // 1 + index of the last valid key of this batch item
+    unsigned rho2_bits;              // max |scaled query|^2 over the workgroup (bits of a non-negative float)
 };
 
 // Exchange between the two half-waves: lane l and lane l^32 hold the same query.
@@ -70,12 +96,22 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
 }
 
-__global__ __launch_bounds__(GA_THREADS)
+// a = h + m + l with h, m, l representable in bf16 (exact for any finite float whose pieces do not underflow)
+__device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
+    h = (float)(__bf16)a;
+    const float r1 = a - h;
+    m = (float)(__bf16)r1;
+    l = (float)(__bf16)(r1 - m);
+}
+
+// FORCE_VALU: evaluate the distances on the vector ALU in every workgroup
+template <bool FORCE_VALU>
+__global__ __launch_bounds__(GA_THREADS, 3)
 void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                          const uint16_t* __restrict__ V, const float* __restrict__ coords,
                          const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                          float* __restrict__ O, float* __restrict__ L,
-                         const int H, const int N)
+                         const int H, const int N, const int ZH)
 {
     __shared__ Smem sm;
 
@@ -85,7 +121,22 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int half = lane >> 5;          // which 4-row group of every 8 accumulator rows
     const int col  = lane & 31;          // accumulator column = query within the wave
 
-    const int zh = blockIdx.y;
+    // Workgroup -> (query tile, batch*head).  Consecutive workgroup ids go round-robin over the
+    // 8 XCDs; keep all query tiles of one (batch, head) on one XCD so that its K and V stay in
+    // that XCD's L2.
+    int zh, qt;
+    {
+        const int id = blockIdx.x;
+        if ((ZH & 7) == 0) {
+            const int per_xcd = ZH >> 3;
+            const int r = id >> 3;
+            zh = (id & 7) + 8 * (r % per_xcd);
+            qt = r / per_xcd;
+        } else {
+            zh = id % ZH;
+            qt = id / ZH;
+        }
+    }
     const int z  = zh / H;
     const int h  = zh - z * H;
     const size_t head_off = (size_t)zh * (size_t)N * GA_D;
@@ -98,26 +149,32 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const float sg = sigma[h];
     // exp(-d^2/(2 sg^2)) = exp2(-(d*cs)^2) with cs = sqrt(log2(e)/2)/sg
     const float cscale = 0.84932180028801907f / sg;
+    // origin of the scaled frame: a query in the middle of this workgroup's tile
+    const int   qmid = min(qt * GA_BM + GA_BM / 2, N - 1);
+    const float ox = cz[3 * qmid], oy = cz[3 * qmid + 1], oz = cz[3 * qmid + 2];
+
+    if (tid == 0) { sm.n_eff = mz ? 0 : N; sm.rho2_bits = 0u; }
+    __syncthreads();
+
+    // ---- this lane's query ----
+    const int  q      = qt * GA_BM + wave * 32 + col;
+    const bool q_in   = q < N;
+    const int  qc     = q_in ? q : N - 1;
+    const bool q_ok   = q_in && !(mz && mz[qc]);
+    const float qx = (cz[3 * qc] - ox) * cscale, qy = (cz[3 * qc + 1] - oy) * cscale, qz = (cz[3 * qc + 2] - oz) * cscale;
+    const float qn2 = qx * qx + qy * qy + qz * qz;
+    atomicMax(&sm.rho2_bits, __builtin_bit_cast(unsigned, qn2));
 
     // ---- 1 + index of the last unpadded key: trailing padded tiles are never visited ----
-    if (tid == 0) sm.n_eff = mz ? 0 : N;
-    __syncthreads();
     if (mz) {
         int last = 0;
         for (int j = tid; j < N; j += GA_THREADS) if (!mz[j]) last = j + 1;
-        // wave maximum, then one LDS atomic per wave
         for (int o = 32; o > 0; o >>= 1) last = max(last, __shfl_xor(last, o));
         if (lane == 0) atomicMax(&sm.n_eff, last);
     }
     __syncthreads();
-    const int n_eff = sm.n_eff;
-
-    // ---- this lane's query ----
-    const int  q      = blockIdx.x * GA_BM + wave * 32 + col;
-    const bool q_in   = q < N;
-    const int  qc     = q_in ? q : N - 1;
-    const bool q_ok   = q_in && !(mz && mz[qc]);
-    const float qx = cz[3 * qc] * cscale, qy = cz[3 * qc + 1] * cscale, qz = cz[3 * qc + 2] * cscale;
+    const int  n_eff = sm.n_eff;
+    const bool use_mfma_dist = !FORCE_VALU && (__builtin_bit_cast(float, sm.rho2_bits) <= GA_MFMA_DIST_MAX_RHO2);
 
     // Q^T as the B operand: lane (half, col) holds d = 16*ks + 8*half + 0..7 of its query,
     // pre-multiplied by 1/sqrt(64) = 2^-3 (exact in bf16)
@@ -129,6 +186,33 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
         qreg[ks] = v;
+    }
+
+    // Query side of the distance contraction.  Slot s of the 24:
+    //   6c+{0..5}, c = x,y,z : key pieces (h,h,m,m,h,l) against query pieces 2*(h,m,h,m,l,h)
+    //   18..20 : key -|x'_k|^2 pieces (h,m,l) against 1
+    //   21..23 : 1 against query -|x'_q|^2 pieces (h,m,l)
+    // First MFMA (K=16): half-wave hf holds slots 8*hf+0..7; second (K=8): slots 16+4*hf+0..3.
+    uint4 gq0;
+    uint2 gq1;
+    {
+        float b[24];
+        const float qs[3] = {qx, qy, qz};
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            float hh, mm, ll;
+            split3(2.0f * qs[c], hh, mm, ll);
+            b[6 * c + 0] = hh; b[6 * c + 1] = mm; b[6 * c + 2] = hh; b[6 * c + 3] = mm; b[6 * c + 4] = ll; b[6 * c + 5] = hh;
+        }
+        b[18] = 1.f; b[19] = 1.f; b[20] = 1.f;
+        split3(-qn2, b[21], b[22], b[23]);
+        float s0[8], s1[4];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s0[e] = half ? b[8 + e] : b[e];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s1[e] = half ? b[20 + e] : b[16 + e];
+        gq0 = make_uint4(pack_bf16(s0[0], s0[1]), pack_bf16(s0[2], s0[3]), pack_bf16(s0[4], s0[5]), pack_bf16(s0[6], s0[7]));
+        gq1 = make_uint2(pack_bf16(s1[0], s1[1]), pack_bf16(s1[2], s1[3]));
     }
 
     floatx16 oacc[2];
@@ -144,99 +228,151 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int vdc  = tid >> 5;   // V: 8-wide d chunk
     const int krow = tid >> 3;   // K: key row (0..31, +32 on the second pass)
     const int kdc  = tid & 7;    // K: 8-wide d chunk
+    const int gkey = tid >> 2;   // geometry: key
+    const int gcmp = tid & 3;    // geometry: x, y, z, -norm^2
 
-    for (int j0 = 0; j0 < n_eff; j0 += GA_BN) {
-        // ---- global -> registers ----
-        uint4 kreg[2], vreg[2];
+    // A key farther than 5 + rho (scaled units) from the origin is at least 5 from every query of
+    // the workgroup: exp2(-25) < 2^-24/2, so s*(1+rbf) rounds to s and the multiplier can be skipped.
+    const float rho       = __builtin_sqrtf(__builtin_bit_cast(float, sm.rho2_bits));
+    const float far_n2    = (5.0f + rho) * (5.0f + rho);
+
+    // registers holding the tile in flight from global memory
+    uint4 kreg[2], vreg[2];
+    float gx = 0.f, gy = 0.f, gz = 0.f;
+    bool  kvalid = false;
+    const uint16_t* kptr = Kh + (size_t)krow * GA_D + kdc * 8;      // advanced by one tile per load
+    const uint16_t* vptr = Vh + (size_t)(2 * kp) * GA_D + vdc * 8;
+    const float*    gptr = cz + 3 * (size_t)gkey;
+
+    auto load_tile = [&](const int j0) {
+        if (j0 + GA_BN <= N) {                 // interior tile: no bounds checks
+            kreg[0] = *reinterpret_cast<const uint4*>(kptr);
+            kreg[1] = *reinterpret_cast<const uint4*>(kptr + 32 * GA_D);
+            vreg[0] = *reinterpret_cast<const uint4*>(vptr);
+            vreg[1] = *reinterpret_cast<const uint4*>(vptr + GA_D);
+            gx = gptr[0]; gy = gptr[1]; gz = gptr[2];
+        } else {
 #pragma unroll
-        for (int p = 0; p < 2; ++p) {
-            const int j = j0 + krow + 32 * p;
-            kreg[p] = (j < N) ? *reinterpret_cast<const uint4*>(Kh + (size_t)j * GA_D + kdc * 8) : make_uint4(0, 0, 0, 0);
-            const int jv = j0 + 2 * kp + p;
-            vreg[p] = (jv < N) ? *reinterpret_cast<const uint4*>(Vh + (size_t)jv * GA_D + vdc * 8) : make_uint4(0, 0, 0, 0);
-        }
-        float kcx = 0.f, kcy = 0.f, kcz = 0.f, kb = 0.f;
-        bool kvalid = false;
-        if (tid < GA_BN) {
-            const int j = j0 + tid;
-            if (j < N) {
-                kcx = cz[3 * j] * cscale; kcy = cz[3 * j + 1] * cscale; kcz = cz[3 * j + 2] * cscale;
-                kvalid = !(mz && mz[j]);
+            for (int p = 0; p < 2; ++p) {
+                kreg[p] = (j0 + krow + 32 * p < N) ? *reinterpret_cast<const uint4*>(kptr + 32 * p * GA_D) : make_uint4(0, 0, 0, 0);
+                vreg[p] = (j0 + 2 * kp + p < N) ? *reinterpret_cast<const uint4*>(vptr + p * GA_D) : make_uint4(0, 0, 0, 0);
             }
-            kb = kvalid ? 0.f : -INFINITY;
+            gx = ox; gy = oy; gz = oz;
+            if (j0 + gkey < N) { gx = gptr[0]; gy = gptr[1]; gz = gptr[2]; }
         }
+        gx = (gx - ox) * cscale; gy = (gy - oy) * cscale; gz = (gz - oz) * cscale;
+        kvalid = true;
+        if (mz || j0 + GA_BN > N) {
+            kvalid = false;
+            if (tid < GA_BN) {
+                const int j = j0 + tid;
+                kvalid = (j < N) && !(mz && mz[j]);
+            }
+        }
+        kptr += GA_BN * GA_D; vptr += GA_BN * GA_D; gptr += 3 * GA_BN;
+    };
 
-        __syncthreads();      // previous tile fully consumed
-        // ---- registers -> LDS ----
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-            *reinterpret_cast<uint4*>(&sm.k[(krow + 32 * p) * GA_LDK + kdc * 8]) = kreg[p];
+    // flags of a tile buffer: [0] has a masked key, [1] has a valid key, [2] == tile number + 1 if the
+    // tile has a key near enough for the multiplier to matter
+    auto store_tile = [&](TileBuf& tb, const int tile_id) {
+        *reinterpret_cast<uint4*>(&tb.k[krow * GA_LDK + kdc * 8]) = kreg[0];
+        *reinterpret_cast<uint4*>(&tb.k[(krow + 32) * GA_LDK + kdc * 8]) = kreg[1];
         {
-            const uint16_t* v0 = reinterpret_cast<const uint16_t*>(&vreg[0]);
-            const uint16_t* v1 = reinterpret_cast<const uint16_t*>(&vreg[1]);
+            const unsigned a[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
+            const unsigned b[4] = {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const unsigned pr = (unsigned)v0[e] | ((unsigned)v1[e] << 16);
-                *reinterpret_cast<unsigned*>(&sm.vt[(vdc * 8 + e) * GA_LDV + 2 * kp]) = pr;
+            for (int e = 0; e < 4; ++e) {
+                // V^T[d][key pair]: low half-word = even key, high half-word = odd key
+                const unsigned lo = __builtin_amdgcn_perm(b[e], a[e], 0x05040100u);
+                const unsigned hi = __builtin_amdgcn_perm(b[e], a[e], 0x07060302u);
+                *reinterpret_cast<unsigned*>(&tb.vt[(vdc * 8 + 2 * e) * GA_LDV + 2 * kp]) = lo;
+                *reinterpret_cast<unsigned*>(&tb.vt[(vdc * 8 + 2 * e + 1) * GA_LDV + 2 * kp]) = hi;
             }
+        }
+        const float n2 = gx * gx + gy * gy + gz * gz;
+        // every wave writes its keys' geometry (a tile is "near" as a whole, so far keys of a near
+        // tile are read too); the flag holds the tile number + 1, so it never needs clearing
+        if (__builtin_amdgcn_ballot_w64(n2 <= far_n2) != 0 && lane == 0) tb.flags[2] = tile_id + 1;
+        if (use_mfma_dist) {
+            // the four threads of a key write the pieces of x, y, z and -|x'|^2 (6 slots = 12 bytes each)
+            const float a = (gcmp == 0) ? gx : (gcmp == 1) ? gy : (gcmp == 2) ? gz : -n2;
+            float hh, mm, ll;
+            split3(a, hh, mm, ll);
+            unsigned w0, w1, w2;
+            if (gcmp < 3) { w0 = pack_bf16(hh, hh); w1 = pack_bf16(mm, mm); w2 = pack_bf16(hh, ll); }
+            else          { w0 = pack_bf16(hh, mm); w1 = pack_bf16(ll, 1.f); w2 = pack_bf16(1.f, 1.f); }
+            unsigned* dst = reinterpret_cast<unsigned*>(&tb.geo[gkey * GA_LDG + 6 * gcmp]);
+            dst[0] = w0; dst[1] = w1; dst[2] = w2;
+        } else if (gcmp == 0) {
+            tb.cx[gkey] = gx; tb.cy[gkey] = gy; tb.cz[gkey] = gz;
         }
         if (tid < GA_BN) {
-            sm.cx[tid] = kcx; sm.cy[tid] = kcy; sm.cz[tid] = kcz; sm.bias[tid] = kb;
+            tb.bias[tid] = kvalid ? 0.f : -INFINITY;
             const uint64_t bal = __builtin_amdgcn_ballot_w64(kvalid);
-            if (tid == 0) { sm.flags[0] = (bal != ~0ull); sm.flags[1] = (bal != 0ull); }
+            if (tid == 0) { tb.flags[0] = (bal != ~0ull); tb.flags[1] = (bal != 0ull); }
         }
-        __syncthreads();
-        const bool has_masked = sm.flags[0] != 0;
-        const bool has_valid  = sm.flags[1] != 0;
-        if (!has_valid) continue;
+    };
 
-        // ---- S^T = K_tile x Q^T : two 32-key blocks ----
-        floatx16 sacc[2];
+    // one 32-key block: S^T, multiplier, mask, online softmax, O^T += V^T x P^T
+    // accumulator register r of block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4)
+    auto block = [&](const TileBuf& tb, const int mt, const bool has_masked, const bool near) {
+        floatx16 sacc;
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[mt][r] = 0.f;
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(&tb.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qreg[ks], sacc, 0, 0, 0);
+        }
+        if (near) {
+            if (use_mfma_dist) {
+                const uint16_t* grow = &tb.geo[(mt * 32 + col) * GA_LDG];
+                const uint4 g0 = *reinterpret_cast<const uint4*>(grow + 8 * half);
+                const uint2 g1 = *reinterpret_cast<const uint2*>(grow + 16 + 4 * half);
+                floatx16 dacc;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const uint4 raw = *reinterpret_cast<const uint4*>(&sm.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
-                sacc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qreg[ks], sacc[mt], 0, 0, 0);
+                for (int r = 0; r < 16; ++r) dacc[r] = 0.f;
+                dacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, g0), __builtin_bit_cast(bf16x8, gq0), dacc, 0, 0, 0);
+                dacc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, g1), __builtin_bit_cast(shortx4, gq1), dacc, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float rbf = __builtin_amdgcn_exp2f(dacc[r]);
+                    sacc[r] = __builtin_fmaf(sacc[r], rbf, sacc[r]);
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int kb0 = mt * 32 + 8 * g + 4 * half;
+                    const float4 kx = *reinterpret_cast<const float4*>(&tb.cx[kb0]);
+                    const float4 ky = *reinterpret_cast<const float4*>(&tb.cy[kb0]);
+                    const float4 kz = *reinterpret_cast<const float4*>(&tb.cz[kb0]);
+                    const float kxs[4] = {kx.x, kx.y, kx.z, kx.w};
+                    const float kys[4] = {ky.x, ky.y, ky.z, ky.w};
+                    const float kzs[4] = {kz.x, kz.y, kz.z, kz.w};
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float dx = qx - kxs[v], dy = qy - kys[v], dz = qz - kzs[v];
+                        const float d2 = dx * dx + dy * dy + dz * dz;
+                        const float rbf = __builtin_amdgcn_exp2f(-d2);
+                        const float sv = sacc[4 * g + v];
+                        sacc[4 * g + v] = __builtin_fmaf(sv, rbf, sv);
+                    }
+                }
             }
         }
-
-        // ---- geometric multiplier, mask, tile maximum ----
-        // accumulator register r of block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4)
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
+        if (has_masked) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int kb0 = mt * 32 + 8 * g + 4 * half;
-                const float4 kx = *reinterpret_cast<const float4*>(&sm.cx[kb0]);
-                const float4 ky = *reinterpret_cast<const float4*>(&sm.cy[kb0]);
-                const float4 kz = *reinterpret_cast<const float4*>(&sm.cz[kb0]);
-                const float kxs[4] = {kx.x, kx.y, kx.z, kx.w};
-                const float kys[4] = {ky.x, ky.y, ky.z, ky.w};
-                const float kzs[4] = {kz.x, kz.y, kz.z, kz.w};
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float dx = qx - kxs[v], dy = qy - kys[v], dz = qz - kzs[v];
-                    const float d2 = dx * dx + dy * dy + dz * dz;
-                    const float rbf = __builtin_amdgcn_exp2f(-d2);
-                    const float s = sacc[mt][4 * g + v];
-                    sacc[mt][4 * g + v] = __builtin_fmaf(s, rbf, s);
-                }
-                if (has_masked) {
-                    const float4 b = *reinterpret_cast<const float4*>(&sm.bias[kb0]);
-                    sacc[mt][4 * g + 0] += b.x; sacc[mt][4 * g + 1] += b.y;
-                    sacc[mt][4 * g + 2] += b.z; sacc[mt][4 * g + 3] += b.w;
-                }
-#pragma unroll
-                for (int v = 0; v < 4; ++v) tmax = fmaxf(tmax, sacc[mt][4 * g + v]);
+                const float4 b = *reinterpret_cast<const float4*>(&tb.bias[mt * 32 + 8 * g + 4 * half]);
+                sacc[4 * g + 0] += b.x; sacc[4 * g + 1] += b.y; sacc[4 * g + 2] += b.z; sacc[4 * g + 3] += b.w;
             }
         }
+        float tmax = sacc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
         tmax = xhalf_max(tmax);
 
-        // ---- online softmax: rescale only when some query's maximum moved ----
+        // online softmax: rescale only when some query's maximum moved
         const float m_new = fmaxf(m_run, tmax);
         if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -250,34 +386,56 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         }
         const float mneg = -((m_run == -INFINITY) ? 0.f : m_run) * LOG2E;
 
-        // ---- P^T (bf16) and O^T += V^T_tile x P^T ----
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-            float p[16];
+        for (int t = 0; t < 2; ++t) {
+            // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
+            float p[8];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], LOG2E, mneg));
-                l_run += p[r];
+            for (int e = 0; e < 8; ++e) {
+                p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t + e], LOG2E, mneg));
+                l_run += p[e];
             }
+            uint4 pb;
+            pb.x = pack_bf16(p[0], p[1]);
+            pb.y = pack_bf16(p[2], p[3]);
+            pb.z = pack_bf16(p[4], p[5]);
+            pb.w = pack_bf16(p[6], p[7]);
+            const int key0 = mt * 32 + 16 * t + 4 * half;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
-                uint4 pb;
-                pb.x = pack_bf16(p[8 * t + 0], p[8 * t + 1]);
-                pb.y = pack_bf16(p[8 * t + 2], p[8 * t + 3]);
-                pb.z = pack_bf16(p[8 * t + 4], p[8 * t + 5]);
-                pb.w = pack_bf16(p[8 * t + 6], p[8 * t + 7]);
-                const int key0 = mt * 32 + 16 * t + 4 * half;
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
-                    const uint16_t* row = &sm.vt[(dt * 32 + col) * GA_LDV + key0];
-                    const uint2 a0 = *reinterpret_cast<const uint2*>(row);
-                    const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
-                    const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb), oacc[dt], 0, 0, 0);
-                }
+            for (int dt = 0; dt < 2; ++dt) {
+                const uint16_t* row = &tb.vt[(dt * 32 + col) * GA_LDV + key0];
+                const uint2 a0 = *reinterpret_cast<const uint2*>(row);
+                const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
+                const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb), oacc[dt], 0, 0, 0);
             }
         }
+    };
+
+    // ---- key loop: tile t is computed from LDS while tile t+1 travels global -> registers -> the other LDS buffer ----
+    const int ntiles = (n_eff + GA_BN - 1) / GA_BN;
+    if (tid == 0) { sm.tile[0].flags[2] = 0; sm.tile[1].flags[2] = 0; }
+    __syncthreads();
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(sm.tile[0], 0);
+        if (ntiles > 1) load_tile(GA_BN);
+    }
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        const TileBuf& tb = sm.tile[t & 1];
+        const bool has_valid  = tb.flags[1] != 0;
+        const bool has_masked = tb.flags[0] != 0;
+        const bool near       = tb.flags[2] == t + 1;
+        if (has_valid) {
+            block(tb, 0, has_masked, near);
+            block(tb, 1, has_masked, near);
+        }
+        if (t + 1 < ntiles) {
+            store_tile(sm.tile[(t + 1) & 1], t + 1);
+            if (t + 2 < ntiles) load_tile((t + 2) * GA_BN);
+        }
+        __syncthreads();
     }
 
     // ---- epilogue ----
@@ -299,7 +457,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 }
 
 struct GaVariant { const char* name; };
-const GaVariant kVariants[] = { {"auto"}, {"w4_q32_k64"} };
+const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -335,8 +493,14 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
     const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
     if (rc != PROTEUS_OK) return rc;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    dim3 grid((N + GA_BM - 1) / GA_BM, Z * H, 1);
-    hipLaunchKernelGGL(geo_attn_fwd_kernel, grid, dim3(GA_THREADS), 0, st,
-                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N);
+    const int n_qtiles = (N + GA_BM - 1) / GA_BM;
+    const int ZH = Z * H;
+    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
+    if (tuning == 2)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<true>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH);
+    else
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<false>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH);
     return (int)hipGetLastError();
 }
