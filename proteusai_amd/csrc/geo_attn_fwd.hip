@@ -5,20 +5,23 @@
 //   s_ij = (q_i . k_j)/sqrt(d) * (1 + exp(-|r_i - r_j|^2 / (2 sigma_h^2))),  -inf for padded keys
 //   O_i  = softmax_j(s_ij) V_j,  L_i = logsumexp_j s_ij;  padded/empty rows -> O = 0, L = -inf
 //
-// Mapping to the machine.  A workgroup is 4 waves; a wave owns 32 queries of one
-// (batch, head) and walks the keys in tiles of 64 that the workgroup stages in
-// LDS (K row-major, V transposed, key geometry).  All products run on the matrix
-// cores and are computed TRANSPOSED:
+// Mapping to the machine.  A workgroup is 4 waves; a wave owns 64 queries of one
+// (batch, head) as two blocks of 32 and walks the keys in tiles of 64 that the
+// workgroup stages in LDS (K row-major, V transposed, key geometry), two tiles
+// deep: tile t is consumed while tile t+1 travels global -> registers -> LDS.
+// All products run on the matrix cores and are computed TRANSPOSED:
 //   S^T (keys x queries)  = K_tile (A, from LDS) x Q^T (B, registers, loaded once)
 //   D^T (keys x queries)  = G_tile (A, from LDS) x G_q^T (B, registers)     [geometry, see below]
 //   O^T (d x queries)    += V^T_tile (A, from LDS) x P^T (B, registers)
 // In the 32x32 accumulator layout a lane holds 16 rows of ONE column, so with
-// queries on the columns each lane owns one query: the row maximum, the
-// exponentials and the row sum are in-lane except for one exchange between the
-// two half-waves, and the S^T accumulator registers are, after conversion to
-// bf16, already the B operand of the last product (the contraction index is
+// queries on the columns each lane owns one query per block: the row maximum,
+// the exponentials and the row sum are in-lane except for one exchange between
+// the two half-waves, and the S^T accumulator registers are, after conversion
+// to bf16, already the B operand of the last product (the contraction index is
 // merely visited in the permuted order the accumulator layout dictates, and the
-// V^T operand is read from LDS in that same order).
+// V^T operand is read from LDS in that same order).  Every A fragment read from
+// LDS serves both query blocks, and the two blocks give the wave independent
+// matrix and vector work to overlap.
 //
 // Geometry on the matrix cores.  With x' = (x - c) * sqrt(log2(e)/2)/sigma_h (c = a
 // point near the workgroup's queries) the multiplier is 1 + exp2(D),
@@ -50,7 +53,8 @@ typedef short  shortx4 __attribute__((ext_vector_type(4)));
 
 constexpr int GA_WAVES   = 4;
 constexpr int GA_THREADS = GA_WAVES * 64;
-constexpr int GA_BM      = GA_WAVES * 32;   // queries per workgroup
+constexpr int GA_QB      = 2;                        // 32-query blocks per wave
+constexpr int GA_BM      = GA_WAVES * 32 * GA_QB;    // queries per workgroup
 constexpr int GA_BN      = 64;              // keys per tile
 constexpr int GA_D       = 64;              // head dim
 constexpr int GA_LDK     = GA_D + 8;        // LDS row stride of the K tile (bf16 elements)
@@ -60,6 +64,8 @@ constexpr float LOG2E    = 1.4426950408889634f;
 // Largest squared distance (scaled units) of a workgroup's queries from their origin for
 // which the matrix-core distance path is used.
 constexpr float GA_MFMA_DIST_MAX_RHO2 = 1000.0f;
+// exp2(-d^2) < 2^-25 for scaled distances d > GA_FAR: s*(1+rbf) then rounds to s in fp32
+constexpr float GA_FAR = 5.0f;
 
 // One staged key tile.  Two of them are kept so that the next tile can be written
 // while the current one is still being read (one barrier per tile).
@@ -70,10 +76,12 @@ struct __align__(16) TileBuf {
     float    cx[GA_BN], cy[GA_BN], cz[GA_BN];   // scaled key coordinates (vector-ALU distance path)
     float    bias[GA_BN];            // 0 for a valid key, -inf for a padded / out-of-range one
     int      flags[4];               // [0] tile has a masked key, [1] tile has a valid key
+    int      near[GA_WAVES];         // == tile number + 1 if a key of the tile can matter to wave w's multiplier
 };
 
 struct __align__(16) Smem {
     TileBuf  tile[2];
+    float4   sphere[GA_WAVES];       // per wave: centre of its queries (scaled frame) and (GA_FAR + radius)^2
     int      n_eff;                  // 1 + index of the last valid key of this batch item
     unsigned rho2_bits;              // max |scaled query|^2 over the workgroup (bits of a non-negative float)
 };
@@ -104,14 +112,17 @@ __device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
     l = (float)(__bf16)(r1 - m);
 }
 
-// FORCE_VALU: evaluate the distances on the vector ALU in every workgroup
-template <bool FORCE_VALU>
-__global__ __launch_bounds__(GA_THREADS, 3)
+// DIST_VALU selects how the distances are evaluated: false = on the matrix cores, true = directly on
+// the vector ALU.  Both instantiations are launched over the same grid; unless take_all is set, a
+// workgroup runs in the matrix-core kernel if its queries lie within GA_MFMA_DIST_MAX_RHO2 of their
+// origin and in the vector-ALU kernel otherwise, and returns at once from the other one.
+template <bool DIST_VALU>
+__global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                          const uint16_t* __restrict__ V, const float* __restrict__ coords,
                          const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                          float* __restrict__ O, float* __restrict__ L,
-                         const int H, const int N, const int ZH)
+                         const int H, const int N, const int ZH, const int take_all)
 {
     __shared__ Smem sm;
 
@@ -119,7 +130,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5;          // which 4-row group of every 8 accumulator rows
-    const int col  = lane & 31;          // accumulator column = query within the wave
+    const int col  = lane & 31;          // accumulator column = query within a block
 
     // Workgroup -> (query tile, batch*head).  Consecutive workgroup ids go round-robin over the
     // 8 XCDs; keep all query tiles of one (batch, head) on one XCD so that its K and V stay in
@@ -156,14 +167,36 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     if (tid == 0) { sm.n_eff = mz ? 0 : N; sm.rho2_bits = 0u; }
     __syncthreads();
 
-    // ---- this lane's query ----
-    const int  q      = qt * GA_BM + wave * 32 + col;
-    const bool q_in   = q < N;
-    const int  qc     = q_in ? q : N - 1;
-    const bool q_ok   = q_in && !(mz && mz[qc]);
-    const float qx = (cz[3 * qc] - ox) * cscale, qy = (cz[3 * qc + 1] - oy) * cscale, qz = (cz[3 * qc + 2] - oz) * cscale;
-    const float qn2 = qx * qx + qy * qy + qz * qz;
-    atomicMax(&sm.rho2_bits, __builtin_bit_cast(unsigned, qn2));
+    // ---- this lane's queries: one per block ----
+    const int qbase = qt * GA_BM + wave * (32 * GA_QB);
+    int   q[GA_QB];
+    bool  q_in[GA_QB], q_ok[GA_QB];
+    float qx[GA_QB], qy[GA_QB], qz[GA_QB], qn2[GA_QB];
+#pragma unroll
+    for (int b = 0; b < GA_QB; ++b) {
+        q[b]    = qbase + 32 * b + col;
+        q_in[b] = q[b] < N;
+        const int qc = q_in[b] ? q[b] : N - 1;
+        q_ok[b] = q_in[b] && !(mz && mz[qc]);
+        qx[b] = (cz[3 * qc] - ox) * cscale; qy[b] = (cz[3 * qc + 1] - oy) * cscale; qz[b] = (cz[3 * qc + 2] - oz) * cscale;
+        qn2[b] = qx[b] * qx[b] + qy[b] * qy[b] + qz[b] * qz[b];
+    }
+    atomicMax(&sm.rho2_bits, __builtin_bit_cast(unsigned, fmaxf(qn2[0], qn2[1])));
+
+    // ---- sphere around this wave's queries, for the far-tile test ----
+    {
+        const int   qw = min(qbase + 32, N - 1);
+        const float wx = (cz[3 * qw] - ox) * cscale, wy = (cz[3 * qw + 1] - oy) * cscale, wz = (cz[3 * qw + 2] - oz) * cscale;
+        float r2 = 0.f;
+#pragma unroll
+        for (int b = 0; b < GA_QB; ++b) {
+            const float dx = qx[b] - wx, dy = qy[b] - wy, dz = qz[b] - wz;
+            r2 = fmaxf(r2, dx * dx + dy * dy + dz * dz);
+        }
+        for (int o = 32; o > 0; o >>= 1) r2 = fmaxf(r2, __shfl_xor(r2, o));
+        const float t = GA_FAR + __builtin_sqrtf(r2) * 1.0001f;
+        if (lane == 0) sm.sphere[wave] = make_float4(wx, wy, wz, t * t);
+    }
 
     // ---- 1 + index of the last unpadded key: trailing padded tiles are never visited ----
     if (mz) {
@@ -174,18 +207,26 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     }
     __syncthreads();
     const int  n_eff = sm.n_eff;
-    const bool use_mfma_dist = !FORCE_VALU && (__builtin_bit_cast(float, sm.rho2_bits) <= GA_MFMA_DIST_MAX_RHO2);
+    constexpr bool use_mfma_dist = !DIST_VALU;
+    if (!take_all) {
+        const bool compact = __builtin_bit_cast(float, sm.rho2_bits) <= GA_MFMA_DIST_MAX_RHO2;
+        if (compact == DIST_VALU) return;       // the other instantiation owns this workgroup
+    }
 
     // Q^T as the B operand: lane (half, col) holds d = 16*ks + 8*half + 0..7 of its query,
     // pre-multiplied by 1/sqrt(64) = 2^-3 (exact in bf16)
-    bf16x8 qreg[4];
+    bf16x8 qreg[GA_QB][4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(Qh + (size_t)qc * GA_D + ks * 16 + half * 8);
-        bf16x8 v = __builtin_bit_cast(bf16x8, raw);
+    for (int b = 0; b < GA_QB; ++b) {
+        const int qc = q_in[b] ? q[b] : N - 1;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
-        qreg[ks] = v;
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(Qh + (size_t)qc * GA_D + ks * 16 + half * 8);
+            bf16x8 v = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
+            qreg[b][ks] = v;
+        }
     }
 
     // Query side of the distance contraction.  Slot s of the 24:
@@ -193,35 +234,37 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     //   18..20 : key -|x'_k|^2 pieces (h,m,l) against 1
     //   21..23 : 1 against query -|x'_q|^2 pieces (h,m,l)
     // First MFMA (K=16): half-wave hf holds slots 8*hf+0..7; second (K=8): slots 16+4*hf+0..3.
-    uint4 gq0;
-    uint2 gq1;
-    {
-        float b[24];
-        const float qs[3] = {qx, qy, qz};
+    uint4 gq0[GA_QB];
+    uint2 gq1[GA_QB];
 #pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            float hh, mm, ll;
-            split3(2.0f * qs[c], hh, mm, ll);
-            b[6 * c + 0] = hh; b[6 * c + 1] = mm; b[6 * c + 2] = hh; b[6 * c + 3] = mm; b[6 * c + 4] = ll; b[6 * c + 5] = hh;
+    for (int b = 0; b < GA_QB; ++b) {
+        float xh, xm, xl, yh, ym, yl, zh_, zm, zl, nh, nm, nl;
+        split3(2.0f * qx[b], xh, xm, xl);
+        split3(2.0f * qy[b], yh, ym, yl);
+        split3(2.0f * qz[b], zh_, zm, zl);
+        split3(-qn2[b], nh, nm, nl);
+        // slots 0..7: x(h,m,h,m,l,h) y(h,m)      slots 8..15: y(h,m,l,h) z(h,m,h,m)
+        // slots 16..19: z(l,h) 1 1                slots 20..23: 1 n(h,m,l)
+        if (half == 0) {
+            gq0[b] = make_uint4(pack_bf16(xh, xm), pack_bf16(xh, xm), pack_bf16(xl, xh), pack_bf16(yh, ym));
+            gq1[b] = make_uint2(pack_bf16(zl, zh_), pack_bf16(1.f, 1.f));
+        } else {
+            gq0[b] = make_uint4(pack_bf16(yh, ym), pack_bf16(yl, yh), pack_bf16(zh_, zm), pack_bf16(zh_, zm));
+            gq1[b] = make_uint2(pack_bf16(1.f, nh), pack_bf16(nm, nl));
         }
-        b[18] = 1.f; b[19] = 1.f; b[20] = 1.f;
-        split3(-qn2, b[21], b[22], b[23]);
-        float s0[8], s1[4];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s0[e] = half ? b[8 + e] : b[e];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s1[e] = half ? b[20 + e] : b[16 + e];
-        gq0 = make_uint4(pack_bf16(s0[0], s0[1]), pack_bf16(s0[2], s0[3]), pack_bf16(s0[4], s0[5]), pack_bf16(s0[6], s0[7]));
-        gq1 = make_uint2(pack_bf16(s1[0], s1[1]), pack_bf16(s1[2], s1[3]));
     }
 
-    floatx16 oacc[2];
+    floatx16 oacc[GA_QB][2];
+    float m_run[GA_QB], l_run[GA_QB];
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int b = 0; b < GA_QB; ++b) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-    float m_run = -INFINITY;     // running maximum of s (natural units), same in both half-waves
-    float l_run = 0.f;           // this half-wave's part of the running sum
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[b][dt][r] = 0.f;
+        m_run[b] = -INFINITY;    // running maximum of s (natural units), same in both half-waves
+        l_run[b] = 0.f;          // this half-wave's part of the running sum
+    }
 
     // staging roles
     const int kp   = tid & 31;   // V: key pair
@@ -229,12 +272,8 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int krow = tid >> 3;   // K: key row (0..31, +32 on the second pass)
     const int kdc  = tid & 7;    // K: 8-wide d chunk
     const int gkey = tid >> 2;   // geometry: key
-    const int gcmp = tid & 3;    // geometry: x, y, z, -norm^2
-
-    // A key farther than 5 + rho (scaled units) from the origin is at least 5 from every query of
-    // the workgroup: exp2(-25) < 2^-24/2, so s*(1+rbf) rounds to s and the multiplier can be skipped.
-    const float rho       = __builtin_sqrtf(__builtin_bit_cast(float, sm.rho2_bits));
-    const float far_n2    = (5.0f + rho) * (5.0f + rho);
+    const int gcmp = tid & 3;    // geometry: x, y, z, -norm^2; far test: against wave gcmp's sphere
+    const float4 sph = sm.sphere[gcmp];
 
     // registers holding the tile in flight from global memory
     uint4 kreg[2], vreg[2];
@@ -272,8 +311,6 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         kptr += GA_BN * GA_D; vptr += GA_BN * GA_D; gptr += 3 * GA_BN;
     };
 
-    // flags of a tile buffer: [0] has a masked key, [1] has a valid key, [2] == tile number + 1 if the
-    // tile has a key near enough for the multiplier to matter
     auto store_tile = [&](TileBuf& tb, const int tile_id) {
         *reinterpret_cast<uint4*>(&tb.k[krow * GA_LDK + kdc * 8]) = kreg[0];
         *reinterpret_cast<uint4*>(&tb.k[(krow + 32) * GA_LDK + kdc * 8]) = kreg[1];
@@ -289,13 +326,20 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 *reinterpret_cast<unsigned*>(&tb.vt[(vdc * 8 + 2 * e + 1) * GA_LDV + 2 * kp]) = hi;
             }
         }
-        const float n2 = gx * gx + gy * gy + gz * gz;
-        // every wave writes its keys' geometry (a tile is "near" as a whole, so far keys of a near
-        // tile are read too); the flag holds the tile number + 1, so it never needs clearing
-        if (__builtin_amdgcn_ballot_w64(n2 <= far_n2) != 0 && lane == 0) tb.flags[2] = tile_id + 1;
+        {
+            // far test of this thread's key against the sphere of wave gcmp; the flag holds the tile
+            // number + 1, so it never needs clearing
+            const float dx = gx - sph.x, dy = gy - sph.y, dz = gz - sph.z;
+            const uint64_t bal = __builtin_amdgcn_ballot_w64(dx * dx + dy * dy + dz * dz <= sph.w);
+            if (lane == 0) {
+#pragma unroll
+                for (int w = 0; w < GA_WAVES; ++w)
+                    if (bal & (0x1111111111111111ull << w)) tb.near[w] = tile_id + 1;
+            }
+        }
         if (use_mfma_dist) {
             // the four threads of a key write the pieces of x, y, z and -|x'|^2 (6 slots = 12 bytes each)
-            const float a = (gcmp == 0) ? gx : (gcmp == 1) ? gy : (gcmp == 2) ? gz : -n2;
+            const float a = (gcmp == 0) ? gx : (gcmp == 1) ? gy : (gcmp == 2) ? gz : -(gx * gx + gy * gy + gz * gz);
             float hh, mm, ll;
             split3(a, hh, mm, ll);
             unsigned w0, w1, w2;
@@ -313,27 +357,12 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         }
     };
 
-    // one 32-key block: S^T, multiplier, mask, online softmax, O^T += V^T x P^T
-    // accumulator register r of block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4)
-    auto block = [&](const TileBuf& tb, const int mt, const bool has_masked, const bool near) {
-        floatx16 sacc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(&tb.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qreg[ks], sacc, 0, 0, 0);
-        }
+    // multiplier, mask, online softmax of one 32-key x 32-query block; returns P^T packed for the two
+    // K=16 steps.  Accumulator register r of key block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4).
+    auto softmax_block = [&](const TileBuf& tb, const int mt, const int b, floatx16& sacc, const floatx16& dacc,
+                             const bool has_masked, const bool near, uint4 (&pb)[2]) {
         if (near) {
             if (use_mfma_dist) {
-                const uint16_t* grow = &tb.geo[(mt * 32 + col) * GA_LDG];
-                const uint4 g0 = *reinterpret_cast<const uint4*>(grow + 8 * half);
-                const uint2 g1 = *reinterpret_cast<const uint2*>(grow + 16 + 4 * half);
-                floatx16 dacc;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) dacc[r] = 0.f;
-                dacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, g0), __builtin_bit_cast(bf16x8, gq0), dacc, 0, 0, 0);
-                dacc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, g1), __builtin_bit_cast(shortx4, gq1), dacc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float rbf = __builtin_amdgcn_exp2f(dacc[r]);
@@ -351,7 +380,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                     const float kzs[4] = {kz.x, kz.y, kz.z, kz.w};
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        const float dx = qx - kxs[v], dy = qy - kys[v], dz = qz - kzs[v];
+                        const float dx = qx[b] - kxs[v], dy = qy[b] - kys[v], dz = qz[b] - kzs[v];
                         const float d2 = dx * dx + dy * dy + dz * dz;
                         const float rbf = __builtin_amdgcn_exp2f(-d2);
                         const float sv = sacc[4 * g + v];
@@ -363,8 +392,8 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         if (has_masked) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const float4 b = *reinterpret_cast<const float4*>(&tb.bias[mt * 32 + 8 * g + 4 * half]);
-                sacc[4 * g + 0] += b.x; sacc[4 * g + 1] += b.y; sacc[4 * g + 2] += b.z; sacc[4 * g + 3] += b.w;
+                const float4 bb = *reinterpret_cast<const float4*>(&tb.bias[mt * 32 + 8 * g + 4 * half]);
+                sacc[4 * g + 0] += bb.x; sacc[4 * g + 1] += bb.y; sacc[4 * g + 2] += bb.z; sacc[4 * g + 3] += bb.w;
             }
         }
         float tmax = sacc[0];
@@ -373,19 +402,19 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         tmax = xhalf_max(tmax);
 
         // online softmax: rescale only when some query's maximum moved
-        const float m_new = fmaxf(m_run, tmax);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+        const float m_new = fmaxf(m_run[b], tmax);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run[b]) != 0) {
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * LOG2E);   // m_run = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f((m_run[b] - m_use) * LOG2E);   // m_run = -inf -> 0
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-            l_run *= alpha;
-            m_run = m_new;
+                for (int r = 0; r < 16; ++r) oacc[b][dt][r] *= alpha;
+            l_run[b] *= alpha;
+            m_run[b] = m_new;
         }
-        const float mneg = -((m_run == -INFINITY) ? 0.f : m_run) * LOG2E;
-
+        const float mneg = -((m_run[b] == -INFINITY) ? 0.f : m_run[b]) * LOG2E;
+        float lsum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
@@ -393,28 +422,67 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t + e], LOG2E, mneg));
-                l_run += p[e];
+                lsum += p[e];
             }
-            uint4 pb;
-            pb.x = pack_bf16(p[0], p[1]);
-            pb.y = pack_bf16(p[2], p[3]);
-            pb.z = pack_bf16(p[4], p[5]);
-            pb.w = pack_bf16(p[6], p[7]);
-            const int key0 = mt * 32 + 16 * t + 4 * half;
+            pb[t] = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+        }
+        l_run[b] += lsum;
+    };
+
+    // one 32-key block of the staged tile against both query blocks
+    auto key_block = [&](const TileBuf& tb, const int mt, const bool has_masked, const bool near) {
+        floatx16 sacc[GA_QB];
+        {
+            uint4 kf[4];
 #pragma unroll
-            for (int dt = 0; dt < 2; ++dt) {
-                const uint16_t* row = &tb.vt[(dt * 32 + col) * GA_LDV + key0];
-                const uint2 a0 = *reinterpret_cast<const uint2*>(row);
-                const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
-                const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb), oacc[dt], 0, 0, 0);
+            for (int ks = 0; ks < 4; ++ks)
+                kf[ks] = *reinterpret_cast<const uint4*>(&tb.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
+#pragma unroll
+            for (int b = 0; b < GA_QB; ++b) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[b][r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+                    sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]), qreg[b][ks], sacc[b], 0, 0, 0);
             }
+        }
+        uint4 g0 = make_uint4(0, 0, 0, 0);
+        uint2 g1 = make_uint2(0, 0);
+        if (near && use_mfma_dist) {
+            const uint16_t* grow = &tb.geo[(mt * 32 + col) * GA_LDG];
+            g0 = *reinterpret_cast<const uint4*>(grow + 8 * half);
+            g1 = *reinterpret_cast<const uint2*>(grow + 16 + 4 * half);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < GA_QB; ++b) {
+            uint4 pb[2];
+            floatx16 dacc;
+            if (near && use_mfma_dist) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dacc[r] = 0.f;
+                dacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, g0), __builtin_bit_cast(bf16x8, gq0[b]), dacc, 0, 0, 0);
+                dacc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, g1), __builtin_bit_cast(shortx4, gq1[b]), dacc, 0, 0, 0);
+            }
+            softmax_block(tb, mt, b, sacc[b], dacc, has_masked, near, pb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) {
+                    const uint16_t* row = &tb.vt[(dt * 32 + col) * GA_LDV + mt * 32 + 16 * t + 4 * half];
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(row);
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
+                    const uint4 vf = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                    oacc[b][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pb[t]), oacc[b][dt], 0, 0, 0);
+                }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
     // ---- key loop: tile t is computed from LDS while tile t+1 travels global -> registers -> the other LDS buffer ----
     const int ntiles = (n_eff + GA_BN - 1) / GA_BN;
-    if (tid == 0) { sm.tile[0].flags[2] = 0; sm.tile[1].flags[2] = 0; }
+    if (tid < GA_WAVES) { sm.tile[0].near[tid] = 0; sm.tile[1].near[tid] = 0; }
     __syncthreads();
     if (ntiles > 0) {
         load_tile(0);
@@ -426,10 +494,10 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         const TileBuf& tb = sm.tile[t & 1];
         const bool has_valid  = tb.flags[1] != 0;
         const bool has_masked = tb.flags[0] != 0;
-        const bool near       = tb.flags[2] == t + 1;
+        const bool near       = tb.near[wave] == t + 1;
         if (has_valid) {
-            block(tb, 0, has_masked, near);
-            block(tb, 1, has_masked, near);
+            key_block(tb, 0, has_masked, near);
+            key_block(tb, 1, has_masked, near);
         }
         if (t + 1 < ntiles) {
             store_tile(sm.tile[(t + 1) & 1], t + 1);
@@ -439,20 +507,23 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     }
 
     // ---- epilogue ----
-    const float l_tot = xhalf_sum(l_run);
-    const bool  row_ok = q_ok && l_tot > 0.f;
-    const float inv_l = row_ok ? 1.0f / l_tot : 0.f;
-    if (q_in) {
-        float* orow = O + head_off + (size_t)q * GA_D;
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
+    for (int b = 0; b < GA_QB; ++b) {
+        const float l_tot = xhalf_sum(l_run[b]);
+        const bool  row_ok = q_ok[b] && l_tot > 0.f;
+        const float inv_l = row_ok ? 1.0f / l_tot : 0.f;
+        if (q_in[b]) {
+            float* orow = O + head_off + (size_t)q[b] * GA_D;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float4 v = make_float4(oacc[dt][4 * g] * inv_l, oacc[dt][4 * g + 1] * inv_l,
-                                       oacc[dt][4 * g + 2] * inv_l, oacc[dt][4 * g + 3] * inv_l);
-                *reinterpret_cast<float4*>(orow + dt * 32 + 8 * g + 4 * half) = v;
-            }
-        if (L && half == 0) L[(size_t)zh * N + q] = row_ok ? m_run + __logf(l_tot) : -INFINITY;
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float4 v = make_float4(oacc[b][dt][4 * g] * inv_l, oacc[b][dt][4 * g + 1] * inv_l,
+                                           oacc[b][dt][4 * g + 2] * inv_l, oacc[b][dt][4 * g + 3] * inv_l);
+                    *reinterpret_cast<float4*>(orow + dt * 32 + 8 * g + 4 * half) = v;
+                }
+            if (L && half == 0) L[(size_t)zh * N + q[b]] = row_ok ? m_run[b] + __logf(l_tot) : -INFINITY;
+        }
     }
 }
 
@@ -496,11 +567,13 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
     const int n_qtiles = (N + GA_BM - 1) / GA_BM;
     const int ZH = Z * H;
     dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
-    if (tuning == 2)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<true>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH);
-    else
+    // tuning 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
+    // 1 / 2: force the matrix-core / vector-ALU path everywhere
+    if (tuning != 2)
         hipLaunchKernelGGL((geo_attn_fwd_kernel<false>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH);
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, tuning == 1 ? 1 : 0);
+    if (tuning != 1)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<true>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, tuning == 2 ? 1 : 0);
     return (int)hipGetLastError();
 }
