@@ -122,7 +122,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                          const uint16_t* __restrict__ V, const float* __restrict__ coords,
                          const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                          float* __restrict__ O, float* __restrict__ L,
-                         const int H, const int N, const int ZH, const int take_all)
+                         const int H, const int N, const int ZH, const int n_qtiles, const int take_all)
 {
     __shared__ Smem sm;
 
@@ -133,8 +133,10 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int col  = lane & 31;          // accumulator column = query within a block
 
     // Workgroup -> (query tile, batch*head).  Consecutive workgroup ids go round-robin over the
-    // 8 XCDs; keep all query tiles of one (batch, head) on one XCD so that its K and V stay in
-    // that XCD's L2.
+    // 8 XCDs.  Each XCD owns ZH/8 (batch, head) pairs for the first half of the query tiles and the
+    // mirrored pairs (ZH-1-zh) for the second half: the K and V an XCD touches at any time stay
+    // few enough for its L2, and a head whose sigma makes the multiplier matter for many tiles is
+    // paired with one for which it matters for few, so the XCDs finish together.
     int zh, qt;
     {
         const int id = blockIdx.x;
@@ -143,6 +145,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             const int r = id >> 3;
             zh = (id & 7) + 8 * (r % per_xcd);
             qt = r / per_xcd;
+            if (2 * qt >= n_qtiles) zh = ZH - 1 - zh;
         } else {
             zh = id % ZH;
             qt = id / ZH;
@@ -571,9 +574,9 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
     // 1 / 2: force the matrix-core / vector-ALU path everywhere
     if (tuning != 2)
         hipLaunchKernelGGL((geo_attn_fwd_kernel<false>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, tuning == 1 ? 1 : 0);
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 1 ? 1 : 0);
     if (tuning != 1)
         hipLaunchKernelGGL((geo_attn_fwd_kernel<true>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, tuning == 2 ? 1 : 0);
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 2 ? 1 : 0);
     return (int)hipGetLastError();
 }
