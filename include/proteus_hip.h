@@ -146,10 +146,11 @@ int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* st
 
 /*
  * Accuracy probe of the hardware sin/cos path used by the WE kernel:
- * s[i] = v_sin_f32(fract(x[i])), c[i] = v_cos_f32(fract(x[i])) with x in
- * revolutions, and q[i] = refined sqrt path r = r2*rsq(r2) applied to x[i].
+ * s[i] = v_sin_f32(y), c[i] = v_cos_f32(y) with x in revolutions and
+ * y = fract(x[i]) if use_fract else x[i] (the instructions accept |y| <= 256),
+ * and q[i] = refined sqrt path r = r2*rsq(r2) applied to x[i].
  */
-int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, void* stream);
+int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, int use_fract, void* stream);
 
 #ifdef __cplusplus
 }

@@ -59,7 +59,7 @@ def load():
     lib.proteus_probe_valu_rate.restype = ci
     lib.proteus_probe_valu_rate.argtypes = [ci, ci, ci, vp, vp]
     lib.proteus_probe_sincos.restype = ci
-    lib.proteus_probe_sincos.argtypes = [vp, vp, vp, vp, ci, vp]
+    lib.proteus_probe_sincos.argtypes = [vp, vp, vp, vp, ci, ci, vp]
     _lib = lib
     return lib
 

@@ -38,11 +38,11 @@ void valu_rate_kernel(float* sink, int iters, float a, float b) {
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
-__global__ void sincos_probe_kernel(const float* x, float* s, float* c, float* q, int n) {
+__global__ void sincos_probe_kernel(const float* x, float* s, float* c, float* q, int n, int use_fract) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float v  = x[i];
-    const float ph = __builtin_amdgcn_fractf(v);
+    const float ph = use_fract ? __builtin_amdgcn_fractf(v) : v;
     s[i] = __builtin_amdgcn_sinf(ph);
     c[i] = __builtin_amdgcn_cosf(ph);
     const float r2 = v;
@@ -89,10 +89,10 @@ extern "C" int proteus_probe_valu_rate(int op, int blocks, int iters, float* sin
     return (int)hipGetLastError();
 }
 
-extern "C" int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, void* stream) {
+extern "C" int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, int use_fract, void* stream) {
     if (!x || !s || !c || !q) return PROTEUS_ERR_NULL_POINTER;
     if (n <= 0) return PROTEUS_ERR_BAD_SHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(sincos_probe_kernel, dim3((n + 255) / 256), dim3(256), 0, st, x, s, c, q, n);
+    hipLaunchKernelGGL(sincos_probe_kernel, dim3((n + 255) / 256), dim3(256), 0, st, x, s, c, q, n, use_fract);
     return (int)hipGetLastError();
 }

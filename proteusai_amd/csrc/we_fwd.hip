@@ -15,8 +15,11 @@
 //     4 wavenumber tiles) stages blocks of source coordinates in LDS, already
 //     compacted to the unpadded ones, and every lane reads the same source with
 //     one broadcast ds_read_b128;
-//   - per (pair, k) the wave issues: v_mul (phase, in revolutions), v_fract,
-//     v_sin, v_cos, 2 x v_fmac (embedding), 2 x v_add (cos/sin sums).
+//   - per (pair, k) the wave issues: v_mul (phase, in revolutions), v_sin, v_cos,
+//     2 x v_fmac (embedding), 2 x v_add (cos/sin sums); v_sin/v_cos take
+//     revolutions and are exact-period for |phase| <= 256, so the explicit range
+//     reduction (v_fract) is issued only for a source whose phase can exceed
+//     that for some lane of the wave (a wave-uniform branch per source).
 // Padded sources never reach the inner loop (compaction), padded observers are
 // computed as ordinary lanes and written as zeros, and the self/coincident pair
 // (r^2 == 0) runs through the loop with r = 0 and 1/r = 0: it adds exactly
@@ -32,24 +35,68 @@ namespace {
 constexpr int WE_WAVES   = 4;
 constexpr int WE_THREADS = WE_WAVES * 64;
 constexpr int WE_JB      = 256;   // sources staged per LDS block (one per thread)
+constexpr float WE_MAX_REV = 250.0f;   // v_sin_f32 / v_cos_f32 accept |x| <= 256 revolutions; keep a margin
 
 __device__ __forceinline__ float sgpr(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
 
+// Inner loop: every lane (observer) against the nk staged sources, KT wavenumbers each.
+// FRACT: reduce the phase to [0,1) revolutions before v_sin/v_cos (needed only when it can exceed
+// the +-256 revolutions those instructions accept).
+template <int KT, bool FRACT>
+__device__ __forceinline__ void stream_sources(const float4* s_keys, const int nk,
+                                               const float xi, const float yi, const float zi,
+                                               const float (&kr)[KT],
+                                               float (&acc_oc)[KT], float (&acc_os)[KT],
+                                               float (&acc_c)[KT], float (&acc_s)[KT], float& nzero)
+{
+    float4 knext = s_keys[0];
+#pragma unroll 1
+    for (int jj = 0; jj < nk; ++jj) {
+        const float4 kj = knext;
+        knext = s_keys[jj + 1];
+        const float dx = xi - kj.x, dy = yi - kj.y, dz = zi - kj.z;
+        const float r2 = dx * dx + dy * dy + dz * dz;
+        const bool  ok = r2 != 0.0f;
+        const float inv = ok ? __builtin_amdgcn_rsqf(r2) : 0.0f;
+        // one Newton step on r = r2 * rsq(r2): r is then within 1 ulp of sqrt(r2)
+        const float r0 = r2 * inv;
+        const float e  = __builtin_fmaf(-r0, r0, r2);
+        const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
+        nzero += ok ? 0.0f : 1.0f;
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            float ph = r * kr[t];
+            if (FRACT) ph = __builtin_amdgcn_fractf(ph);
+            const float s = __builtin_amdgcn_sinf(ph);
+            const float c = __builtin_amdgcn_cosf(ph);
+            acc_oc[t] = __builtin_fmaf(c, inv, acc_oc[t]);
+            acc_os[t] = __builtin_fmaf(s, inv, acc_os[t]);
+            acc_c[t] += c;
+            acc_s[t] += s;
+        }
+    }
+}
+
 // KT     wavenumbers per wave (4*KT accumulators per lane)
 // SPLIT  the sources are split over gridDim.x/ceil(N/64) workgroups and partial
 //        sums are added to pre-zeroed outputs with float atomics (small N only)
-template <int KT, bool SPLIT>
+// FRACT  this instantiation reduces the phase explicitly.  Both instantiations are launched over the
+//        same grid; a workgroup runs in the FRACT=false kernel if no phase of its waves can leave
+//        +-WE_MAX_REV revolutions and in the FRACT=true kernel otherwise (it returns at once from
+//        the other one), unless take_all forces one kernel to take every workgroup.
+template <int KT, bool SPLIT, bool FRACT>
 __global__ __launch_bounds__(WE_THREADS)
 void we_fwd_kernel(const float* __restrict__ coords, const int layout,
                    const float* __restrict__ wavenumbers,
                    const uint8_t* __restrict__ mask,
                    float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
-                   const int N, const int K, const int nsplit)
+                   const int N, const int K, const int nsplit, const int take_all)
 {
     __shared__ float4 s_keys[WE_JB + 1];   // +1: the stream loop reads one source ahead
     __shared__ int    s_wcount[WE_WAVES];
+    __shared__ float  s_box[WE_WAVES][6];
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -85,6 +132,46 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
         const int k = k0 + t;
         const float w = (k < K) ? wavenumbers[k] : 0.0f;
         kr[t] = sgpr((float)((double)w * 0.15915494309189533577));
+    }
+    float kr_max = 0.f;
+#pragma unroll
+    for (int t = 0; t < KT; ++t) kr_max = fmaxf(kr_max, fabsf(kr[t]));
+
+    // ---- can any phase of this wave leave the +-256 revolutions v_sin/v_cos accept? ----
+    // Bounding box of all coordinates of the batch item (a few loads per thread, once), then the
+    // distance from each observer to its farthest corner bounds every r_ij of the lane.
+    {
+        float lo[3] = {3.0e38f, 3.0e38f, 3.0e38f}, hi[3] = {-3.0e38f, -3.0e38f, -3.0e38f};
+        for (int j = tid; j < N; j += WE_THREADS) {
+            float p[3];
+            if (layout == PROTEUS_COORDS_SOA) { p[0] = cz[j]; p[1] = cz[(size_t)N + j]; p[2] = cz[2 * (size_t)N + j]; }
+            else                              { p[0] = cz[3 * (size_t)j]; p[1] = cz[3 * (size_t)j + 1]; p[2] = cz[3 * (size_t)j + 2]; }
+#pragma unroll
+            for (int c = 0; c < 3; ++c) { lo[c] = fminf(lo[c], p[c]); hi[c] = fmaxf(hi[c], p[c]); }
+        }
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+            for (int o = 32; o > 0; o >>= 1) { lo[c] = fminf(lo[c], __shfl_xor(lo[c], o)); hi[c] = fmaxf(hi[c], __shfl_xor(hi[c], o)); }
+        if (lane == 0) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) { s_box[wave][c] = lo[c]; s_box[wave][3 + c] = hi[c]; }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            lo[c] = fminf(fminf(s_box[0][c], s_box[1][c]), fminf(s_box[2][c], s_box[3][c]));
+            hi[c] = fmaxf(fmaxf(s_box[0][3 + c], s_box[1][3 + c]), fmaxf(s_box[2][3 + c], s_box[3][3 + c]));
+        }
+        const float fx = fmaxf(fabsf(xi - lo[0]), fabsf(xi - hi[0]));
+        const float fy = fmaxf(fabsf(yi - lo[1]), fabsf(yi - hi[1]));
+        const float fz = fmaxf(fabsf(zi - lo[2]), fabsf(zi - hi[2]));
+        const float rfar = __builtin_sqrtf(fx * fx + fy * fy + fz * fz);
+        // NaN-safe: anything that is not provably below the limit takes the reducing path
+        const bool wave_safe = __builtin_amdgcn_ballot_w64(!(rfar * kr_max < WE_MAX_REV)) == 0;
+        if (lane == 0) s_wcount[wave] = wave_safe ? 1 : 0;
+        __syncthreads();
+        const bool wg_safe = (s_wcount[0] & s_wcount[1] & s_wcount[2] & s_wcount[3]) != 0;
+        if (!take_all && wg_safe == FRACT) return;      // the other instantiation owns this workgroup
     }
 
     float acc_oc[KT], acc_os[KT], acc_c[KT], acc_s[KT];
@@ -126,31 +213,7 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
             if (!wave_active) continue;
 
             // -- stream the staged sources --
-            float4 knext = s_keys[0];
-#pragma unroll 1
-            for (int jj = 0; jj < nk; ++jj) {
-                const float4 kj = knext;
-                knext = s_keys[jj + 1];
-                const float dx = xi - kj.x, dy = yi - kj.y, dz = zi - kj.z;
-                const float r2 = dx * dx + dy * dy + dz * dz;
-                const bool  ok = r2 != 0.0f;
-                const float inv = ok ? __builtin_amdgcn_rsqf(r2) : 0.0f;
-                // one Newton step on r = r2 * rsq(r2): r is then within 1 ulp of sqrt(r2)
-                const float r0 = r2 * inv;
-                const float e  = __builtin_fmaf(-r0, r0, r2);
-                const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
-                nzero += ok ? 0.0f : 1.0f;
-#pragma unroll
-                for (int t = 0; t < KT; ++t) {
-                    const float ph = __builtin_amdgcn_fractf(r * kr[t]);
-                    const float s  = __builtin_amdgcn_sinf(ph);
-                    const float c  = __builtin_amdgcn_cosf(ph);
-                    acc_oc[t] = __builtin_fmaf(c, inv, acc_oc[t]);
-                    acc_os[t] = __builtin_fmaf(s, inv, acc_os[t]);
-                    acc_c[t] += c;
-                    acc_s[t] += s;
-                }
-            }
+            stream_sources<KT, FRACT>(s_keys, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
         }
     }
 
@@ -221,23 +284,27 @@ void zero_async(float* p, size_t n, hipStream_t st) {
                        reinterpret_cast<float4*>(p), n4, p + n4 * 4, ntail);
 }
 
-struct WeVariant { const char* name; int kt; bool split; };
+// fract: 0 = each workgroup picks (two cooperating launches), 1 = always reduce, -1 = never reduce
+// (only valid when every phase is known to stay within +-256 revolutions; a measuring aid)
+struct WeVariant { const char* name; int kt; bool split; int fract; };
 // index 0 is "automatic"; the others force a tile
 const WeVariant kVariants[] = {
-    {"auto", 0, false},
-    {"kt32", 32, false},
-    {"kt16", 16, false},
-    {"kt8", 8, false},
-    {"kt64", 64, false},
-    {"kt32_split", 32, true},
-    {"kt16_split", 16, true},
-    {"kt8_split", 8, true},
+    {"auto", 0, false, 0},
+    {"kt32", 32, false, 0},
+    {"kt16", 16, false, 0},
+    {"kt8", 8, false, 0},
+    {"kt64", 64, false, 0},
+    {"kt32_split", 32, true, 0},
+    {"kt16_split", 16, true, 0},
+    {"kt8_split", 8, true, 0},
+    {"kt32_fract", 32, false, 1},
+    {"kt32_nofract_unchecked", 32, false, -1},
 };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 template <int KT, bool SPLIT>
 int launch(const float* coords, int layout, const float* wn, const uint8_t* mask,
-           float* out, float* cs, float* ss, int Z, int N, int K, int nsplit, hipStream_t st)
+           float* out, float* cs, float* ss, int Z, int N, int K, int nsplit, int fract, hipStream_t st)
 {
     const int iblocks = (N + 63) / 64;
     const int ktiles  = (K + KT * WE_WAVES - 1) / (KT * WE_WAVES);
@@ -247,8 +314,12 @@ int launch(const float* coords, int layout, const float* wn, const uint8_t* mask
         zero_async(ss,  (size_t)Z * N * K, st);
     }
     dim3 grid(iblocks * (SPLIT ? nsplit : 1), ktiles, Z);
-    hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT>), grid, dim3(WE_THREADS), 0, st,
-                       coords, layout, wn, mask, out, cs, ss, N, K, nsplit);
+    if (fract <= 0)
+        hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT, false>), grid, dim3(WE_THREADS), 0, st,
+                           coords, layout, wn, mask, out, cs, ss, N, K, nsplit, fract < 0 ? 1 : 0);
+    if (fract >= 0)
+        hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT, true>), grid, dim3(WE_THREADS), 0, st,
+                           coords, layout, wn, mask, out, cs, ss, N, K, nsplit, fract > 0 ? 1 : 0);
     return (int)hipGetLastError();
 }
 
@@ -286,6 +357,7 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
 
     int kt = kVariants[tuning].kt;
     bool split = kVariants[tuning].split;
+    const int fract = kVariants[tuning].fract;
     const long iblocks = ((long)N + 63) / 64 * Z;
     if (tuning == 0) {
         // Aim for at least two waves on each of the 1024 SIMDs; prefer the
@@ -304,10 +376,10 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
         if (nsplit > maxsplit) nsplit = maxsplit;
         if (nsplit < 1) nsplit = 1;
     }
-#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, nsplit, st) \
-                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, st))
+#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, nsplit, fract, st) \
+                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, fract, st))
     switch (kt) {
-        case 64: return launch<64, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, st);
+        case 64: return launch<64, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, fract, st);
         case 32: return WE_GO(32);
         case 16: return WE_GO(16);
         default: return WE_GO(8);

@@ -257,3 +257,29 @@ def test_cfg4_batch_with_padding(gpu):
     got = run_gpu(gpu, coords, wn, mask)
     rows = np.sort(np.random.default_rng(4).choice(1024, 64, replace=False)).astype(np.int32)
     check(got, coords, wn, mask, rows=rows, what="cfg4")
+
+
+def test_hardware_sincos_and_sqrt_error(gpu):
+    # the stated fp32 error of the fast path: v_sin_f32 / v_cos_f32 on revolutions, with and without the
+    # explicit range reduction, and r = r2*rsq(r2) with one Newton step
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(0)
+    n = 1 << 20
+    x = ((torch.rand(n, generator=g, dtype=torch.float64) - 0.5) * 500.0).float()      # |x| < 250 revolutions
+    xd = x.to(gpu)
+    s, c, q = torch.empty_like(xd), torch.empty_like(xd), torch.empty_like(xd)
+    ph = 2 * np.pi * (x.double().numpy() % 1.0)
+    for use_fract in (1, 0):
+        rc = lib.proteus_probe_sincos(xd.data_ptr(), s.data_ptr(), c.data_ptr(), q.data_ptr(), n, use_fract, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        es = np.abs(s.cpu().numpy() - np.sin(ph)).max()
+        ec = np.abs(c.cpu().numpy() - np.cos(ph)).max()
+        assert es < 5e-7 and ec < 5e-7, (use_fract, es, ec)
+    r2 = (torch.rand(n, generator=g, dtype=torch.float64) * 1e6).float()
+    rd = r2.to(gpu)
+    rc = lib.proteus_probe_sincos(rd.data_ptr(), s.data_ptr(), c.data_ptr(), q.data_ptr(), n, 1, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = np.sqrt(r2.double().numpy())
+    assert (np.abs(q.cpu().numpy() - ref) / np.maximum(ref, 1e-30)).max() < 1.2e-7
