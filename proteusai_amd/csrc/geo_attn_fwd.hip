@@ -276,23 +276,27 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int kdc  = tid & 7;    // K: 8-wide d chunk
     const int gkey = tid >> 2;   // geometry: key
     const int gcmp = tid & 3;    // geometry: x, y, z, -norm^2; far test: against wave gcmp's sphere
-    const float4 sph = sm.sphere[gcmp];
 
-    // registers holding the tile in flight from global memory
+    // registers holding the tile in flight from global memory.  load_tile only ISSUES loads; nothing
+    // it fetches is touched until store_tile, one tile of computation later, so the wait for them
+    // lands there.
     uint4 kreg[2], vreg[2];
-    float gx = 0.f, gy = 0.f, gz = 0.f;
-    bool  kvalid = false;
+    float gx = 0.f, gy = 0.f, gz = 0.f;     // raw key coordinates
+    unsigned mbyte = 0;                     // raw padding byte of key tid (threads < 64)
+    bool loaded_edge = false;               // the tile in flight is the (partial) last one
     const uint16_t* kptr = Kh + (size_t)krow * GA_D + kdc * 8;      // advanced by one tile per load
     const uint16_t* vptr = Vh + (size_t)(2 * kp) * GA_D + vdc * 8;
     const float*    gptr = cz + 3 * (size_t)gkey;
 
     auto load_tile = [&](const int j0) {
+        loaded_edge = j0 + GA_BN > N;
         if (j0 + GA_BN <= N) {                 // interior tile: no bounds checks
             kreg[0] = *reinterpret_cast<const uint4*>(kptr);
             kreg[1] = *reinterpret_cast<const uint4*>(kptr + 32 * GA_D);
             vreg[0] = *reinterpret_cast<const uint4*>(vptr);
             vreg[1] = *reinterpret_cast<const uint4*>(vptr + GA_D);
             gx = gptr[0]; gy = gptr[1]; gz = gptr[2];
+            if (mz && tid < GA_BN) mbyte = mz[j0 + tid];
         } else {
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
@@ -301,20 +305,15 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             }
             gx = ox; gy = oy; gz = oz;
             if (j0 + gkey < N) { gx = gptr[0]; gy = gptr[1]; gz = gptr[2]; }
-        }
-        gx = (gx - ox) * cscale; gy = (gy - oy) * cscale; gz = (gz - oz) * cscale;
-        kvalid = true;
-        if (mz || j0 + GA_BN > N) {
-            kvalid = false;
-            if (tid < GA_BN) {
-                const int j = j0 + tid;
-                kvalid = (j < N) && !(mz && mz[j]);
-            }
+            mbyte = 1;
+            if (tid < GA_BN && j0 + tid < N) mbyte = mz ? mz[j0 + tid] : 0;
         }
         kptr += GA_BN * GA_D; vptr += GA_BN * GA_D; gptr += 3 * GA_BN;
     };
 
     auto store_tile = [&](TileBuf& tb, const int tile_id) {
+        gx = (gx - ox) * cscale; gy = (gy - oy) * cscale; gz = (gz - oz) * cscale;
+        const bool kvalid = (mz || loaded_edge) ? (mbyte == 0) : true;
         *reinterpret_cast<uint4*>(&tb.k[krow * GA_LDK + kdc * 8]) = kreg[0];
         *reinterpret_cast<uint4*>(&tb.k[(krow + 32) * GA_LDK + kdc * 8]) = kreg[1];
         {
@@ -332,6 +331,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         {
             // far test of this thread's key against the sphere of wave gcmp; the flag holds the tile
             // number + 1, so it never needs clearing
+            const float4 sph = sm.sphere[gcmp];
             const float dx = gx - sph.x, dy = gy - sph.y, dz = gz - sph.z;
             const uint64_t bal = __builtin_amdgcn_ballot_w64(dx * dx + dy * dy + dz * dz <= sph.w);
             if (lane == 0) {
