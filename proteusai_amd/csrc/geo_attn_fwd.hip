@@ -456,7 +456,6 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             g0 = *reinterpret_cast<const uint4*>(grow + 8 * half);
             g1 = *reinterpret_cast<const uint2*>(grow + 16 + 4 * half);
         }
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < GA_QB; ++b) {
             uint4 pb[2];
@@ -468,8 +467,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 dacc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, g1), __builtin_bit_cast(shortx4, gq1[b]), dacc, 0, 0, 0);
             }
             softmax_block(tb, mt, b, sacc[b], dacc, has_masked, near, pb);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
+    #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt) {
@@ -479,8 +477,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                     const uint4 vf = make_uint4(a0.x, a0.y, a1.x, a1.y);
                     oacc[b][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pb[t]), oacc[b][dt], 0, 0, 0);
                 }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+            }
     };
 
     // ---- key loop: tile t is computed from LDS while tile t+1 travels global -> registers -> the other LDS buffer ----
