@@ -50,6 +50,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float  floatx16 __attribute__((ext_vector_type(16)));
 typedef float  floatx2 __attribute__((ext_vector_type(2)));
 typedef short  shortx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uint4v __attribute__((ext_vector_type(4)));
 
 constexpr int GA_WAVES   = 4;
 constexpr int GA_THREADS = GA_WAVES * 64;
@@ -84,6 +85,7 @@ struct __align__(16) Smem {
     float4   sphere[GA_WAVES];       // per wave: centre of its queries (scaled frame) and (GA_FAR + radius)^2
     int      n_eff;                  // 1 + index of the last valid key of this batch item
     unsigned rho2_bits;              // max |scaled query|^2 over the workgroup (bits of a non-negative float)
+    int      q_first, q_last;        // first / last unpadded query of the workgroup
 };
 
 // Exchange between the two half-waves: lane l and lane l^32 hold the same query.
@@ -163,24 +165,56 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const float sg = sigma[h];
     // exp(-d^2/(2 sg^2)) = exp2(-(d*cs)^2) with cs = sqrt(log2(e)/2)/sg
     const float cscale = 0.84932180028801907f / sg;
-    // origin of the scaled frame: a query in the middle of this workgroup's tile
-    const int   qmid = min(qt * GA_BM + GA_BM / 2, N - 1);
-    const float ox = cz[3 * qmid], oy = cz[3 * qmid + 1], oz = cz[3 * qmid + 2];
-
-    if (tid == 0) { sm.n_eff = mz ? 0 : N; sm.rho2_bits = 0u; }
+    if (tid == 0) { sm.n_eff = mz ? 0 : N; sm.rho2_bits = 0u; sm.q_first = 0x7fffffff; sm.q_last = -1; }
     __syncthreads();
 
     // ---- this lane's queries: one per block ----
     const int qbase = qt * GA_BM + wave * (32 * GA_QB);
     int   q[GA_QB];
     bool  q_in[GA_QB], q_ok[GA_QB];
-    float qx[GA_QB], qy[GA_QB], qz[GA_QB], qn2[GA_QB];
 #pragma unroll
     for (int b = 0; b < GA_QB; ++b) {
         q[b]    = qbase + 32 * b + col;
         q_in[b] = q[b] < N;
-        const int qc = q_in[b] ? q[b] : N - 1;
-        q_ok[b] = q_in[b] && !(mz && mz[qc]);
+        q_ok[b] = q_in[b] && !(mz && mz[q[b]]);
+    }
+    // first and last unpadded query of the workgroup (wave-level reduction, then one LDS atomic each)
+    int wave_first, wave_last;
+    {
+        int lo = q_ok[0] ? q[0] : (q_ok[1] ? q[1] : 0x7fffffff);
+        int hi = q_ok[1] ? q[1] : (q_ok[0] ? q[0] : -1);
+        for (int o = 32; o > 0; o >>= 1) { lo = min(lo, __shfl_xor(lo, o)); hi = max(hi, __shfl_xor(hi, o)); }
+        if (lane == 0) { atomicMin(&sm.q_first, lo); atomicMax(&sm.q_last, hi); }
+        wave_first = lo; wave_last = hi;
+    }
+    __syncthreads();
+    const int q_first = sm.q_first, q_last = sm.q_last;
+    if (q_last < 0) {
+        // every query of this workgroup is padded (or out of range): zeros, L = -inf, done
+        if (take_all || DIST_VALU) {      // exactly one of the cooperating kernels writes them
+#pragma unroll
+            for (int b = 0; b < GA_QB; ++b) {
+                if (!q_in[b]) continue;
+                float* orow = O + head_off + (size_t)q[b] * GA_D;
+#pragma unroll
+                for (int g = 0; g < 8; ++g)
+                    *reinterpret_cast<float4*>(orow + 8 * g + 4 * half) = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (L && half == 0) L[(size_t)zh * N + q[b]] = -INFINITY;
+            }
+        }
+        return;
+    }
+    // Origin of the scaled frame: midway between the first and the last unpadded query of the
+    // workgroup.  Only unpadded tokens enter it (and the radius below), so whatever sits in padded
+    // positions cannot change which code path, and hence which rounding, the valid rows see.
+    const float ox = 0.5f * (cz[3 * q_first] + cz[3 * q_last]);
+    const float oy = 0.5f * (cz[3 * q_first + 1] + cz[3 * q_last + 1]);
+    const float oz = 0.5f * (cz[3 * q_first + 2] + cz[3 * q_last + 2]);
+    const int q_mirror = (wave_first != 0x7fffffff) ? wave_first : q_first;
+    float qx[GA_QB], qy[GA_QB], qz[GA_QB], qn2[GA_QB];
+#pragma unroll
+    for (int b = 0; b < GA_QB; ++b) {
+        const int qc = q_ok[b] ? q[b] : q_mirror;      // a padded lane mirrors a valid query: finite, in-range data
         qx[b] = (cz[3 * qc] - ox) * cscale; qy[b] = (cz[3 * qc + 1] - oy) * cscale; qz[b] = (cz[3 * qc + 2] - oz) * cscale;
         qn2[b] = qx[b] * qx[b] + qy[b] * qy[b] + qz[b] * qz[b];
     }
@@ -188,8 +222,11 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 
     // ---- sphere around this wave's queries, for the far-tile test ----
     {
-        const int   qw = min(qbase + 32, N - 1);
-        const float wx = (cz[3 * qw] - ox) * cscale, wy = (cz[3 * qw + 1] - oy) * cscale, wz = (cz[3 * qw + 2] - oz) * cscale;
+        // centre: midway between the wave's first and last unpadded query (the workgroup's, if it has none)
+        const int   qa = q_mirror, qb = (wave_last >= 0) ? wave_last : q_first;
+        const float wx = (0.5f * (cz[3 * qa] + cz[3 * qb]) - ox) * cscale;
+        const float wy = (0.5f * (cz[3 * qa + 1] + cz[3 * qb + 1]) - oy) * cscale;
+        const float wz = (0.5f * (cz[3 * qa + 2] + cz[3 * qb + 2]) - oz) * cscale;
         float r2 = 0.f;
 #pragma unroll
         for (int b = 0; b < GA_QB; ++b) {
@@ -221,7 +258,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     bf16x8 qreg[GA_QB][4];
 #pragma unroll
     for (int b = 0; b < GA_QB; ++b) {
-        const int qc = q_in[b] ? q[b] : N - 1;
+        const int qc = q_ok[b] ? q[b] : q_mirror;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const uint4 raw = *reinterpret_cast<const uint4*>(Qh + (size_t)qc * GA_D + ks * 16 + half * 8);
@@ -279,46 +316,62 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 
     // registers holding the tile in flight from global memory.  load_tile only ISSUES loads; nothing
     // it fetches is touched until store_tile, one tile of computation later, so the wait for them
-    // lands there.
-    uint4 kreg[2], vreg[2];
-    float gx = 0.f, gy = 0.f, gz = 0.f;     // raw key coordinates
+    // lands there.  Buffer loads: base in SGPRs, one 32-bit lane offset, and reads past the end of a
+    // tensor return zeros (no bounds branches on the last tile).
+    uint4v kreg[2], vreg[2];
+    uint4v graw = {0u, 0u, 0u, 0u};         // raw key coordinates (x, y, z and one dword beyond)
     unsigned mbyte = 0;                     // raw padding byte of key tid (threads < 64)
-    bool loaded_edge = false;               // the tile in flight is the (partial) last one
-    const uint16_t* kptr = Kh + (size_t)krow * GA_D + kdc * 8;      // advanced by one tile per load
-    const uint16_t* vptr = Vh + (size_t)(2 * kp) * GA_D + vdc * 8;
-    const float*    gptr = cz + 3 * (size_t)gkey;
+    unsigned mk0 = 0, mk1 = 0, mv0 = 0, mv1 = 0, mg = 0;   // raw padding bytes of the keys this thread stages
+    int loaded_j0 = 0;
+    const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)Kh, 0, N * GA_D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)Vh, 0, N * GA_D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rC = __builtin_amdgcn_make_buffer_rsrc((void*)cz, 0, N * 12, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rM = __builtin_amdgcn_make_buffer_rsrc((void*)(mz ? mz : key_pad), 0, mz ? N : 0, 0x00020000);
+    const int koff = (krow * GA_D + kdc * 8) * 2;            // byte offsets inside a tile
+    const int voff = (2 * kp * GA_D + vdc * 8) * 2;
+    const int goff = 12 * gkey;
 
     auto load_tile = [&](const int j0) {
-        loaded_edge = j0 + GA_BN > N;
-        if (j0 + GA_BN <= N) {                 // interior tile: no bounds checks
-            kreg[0] = *reinterpret_cast<const uint4*>(kptr);
-            kreg[1] = *reinterpret_cast<const uint4*>(kptr + 32 * GA_D);
-            vreg[0] = *reinterpret_cast<const uint4*>(vptr);
-            vreg[1] = *reinterpret_cast<const uint4*>(vptr + GA_D);
-            gx = gptr[0]; gy = gptr[1]; gz = gptr[2];
-            if (mz && tid < GA_BN) mbyte = mz[j0 + tid];
-        } else {
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                kreg[p] = (j0 + krow + 32 * p < N) ? *reinterpret_cast<const uint4*>(kptr + 32 * p * GA_D) : make_uint4(0, 0, 0, 0);
-                vreg[p] = (j0 + 2 * kp + p < N) ? *reinterpret_cast<const uint4*>(vptr + p * GA_D) : make_uint4(0, 0, 0, 0);
-            }
-            gx = ox; gy = oy; gz = oz;
-            if (j0 + gkey < N) { gx = gptr[0]; gy = gptr[1]; gz = gptr[2]; }
-            mbyte = 1;
-            if (tid < GA_BN && j0 + tid < N) mbyte = mz ? mz[j0 + tid] : 0;
+        loaded_j0 = j0;
+        // the tile offset goes into the lane offset, not the scalar offset: only the former is range-checked
+        const int tile_bytes = j0 * GA_D * 2;
+        kreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + tile_bytes, 0, 0);
+        kreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + tile_bytes + 32 * GA_D * 2, 0, 0);
+        vreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + tile_bytes, 0, 0);
+        vreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + tile_bytes + GA_D * 2, 0, 0);
+        graw    = __builtin_amdgcn_raw_buffer_load_b128(rC, goff + j0 * 12, 0, 0);
+        if (mz) {
+            mbyte = __builtin_amdgcn_raw_buffer_load_b8(rM, lane + j0, 0, 0);      // used by wave 0 only
+            mk0 = __builtin_amdgcn_raw_buffer_load_b8(rM, krow + j0, 0, 0);
+            mk1 = __builtin_amdgcn_raw_buffer_load_b8(rM, krow + 32 + j0, 0, 0);
+            mv0 = __builtin_amdgcn_raw_buffer_load_b8(rM, 2 * kp + j0, 0, 0);
+            mv1 = __builtin_amdgcn_raw_buffer_load_b8(rM, 2 * kp + 1 + j0, 0, 0);
+            mg  = __builtin_amdgcn_raw_buffer_load_b8(rM, gkey + j0, 0, 0);
         }
-        kptr += GA_BN * GA_D; vptr += GA_BN * GA_D; gptr += 3 * GA_BN;
     };
 
     auto store_tile = [&](TileBuf& tb, const int tile_id) {
-        gx = (gx - ox) * cscale; gy = (gy - oy) * cscale; gz = (gz - oz) * cscale;
-        const bool kvalid = (mz || loaded_edge) ? (mbyte == 0) : true;
-        *reinterpret_cast<uint4*>(&tb.k[krow * GA_LDK + kdc * 8]) = kreg[0];
-        *reinterpret_cast<uint4*>(&tb.k[(krow + 32) * GA_LDK + kdc * 8]) = kreg[1];
+        // (elements are copied to scalars first: bit-casting a vector element expression directly reads element 0)
+        const unsigned rx = graw[0], ry = graw[1], rz = graw[2];
+        float gx = (__builtin_bit_cast(float, rx) - ox) * cscale;
+        float gy = (__builtin_bit_cast(float, ry) - oy) * cscale;
+        float gz = (__builtin_bit_cast(float, rz) - oz) * cscale;
+        if (mz) {
+            // whatever a padded key holds (even NaN) is replaced by zeros: everything downstream stays
+            // finite and the -inf bias alone removes the key
+            if (mk0) kreg[0] = uint4v{0u, 0u, 0u, 0u};
+            if (mk1) kreg[1] = uint4v{0u, 0u, 0u, 0u};
+            if (mv0) vreg[0] = uint4v{0u, 0u, 0u, 0u};
+            if (mv1) vreg[1] = uint4v{0u, 0u, 0u, 0u};
+            if (mg) { gx = 0.f; gy = 0.f; gz = 0.f; }
+        }
+        if (loaded_j0 + gkey >= N) { gx = 0.f; gy = 0.f; gz = 0.f; }
+        const bool kvalid = (loaded_j0 + tid < N) && (mbyte == 0);
+        *reinterpret_cast<uint4v*>(&tb.k[krow * GA_LDK + kdc * 8]) = kreg[0];
+        *reinterpret_cast<uint4v*>(&tb.k[(krow + 32) * GA_LDK + kdc * 8]) = kreg[1];
         {
-            const unsigned a[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
-            const unsigned b[4] = {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w};
+            const unsigned a[4] = {vreg[0][0], vreg[0][1], vreg[0][2], vreg[0][3]};
+            const unsigned b[4] = {vreg[1][0], vreg[1][1], vreg[1][2], vreg[1][3]};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 // V^T[d][key pair]: low half-word = even key, high half-word = odd key
@@ -518,8 +571,9 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    float4 v = make_float4(oacc[b][dt][4 * g] * inv_l, oacc[b][dt][4 * g + 1] * inv_l,
-                                           oacc[b][dt][4 * g + 2] * inv_l, oacc[b][dt][4 * g + 3] * inv_l);
+                    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (row_ok) v = make_float4(oacc[b][dt][4 * g] * inv_l, oacc[b][dt][4 * g + 1] * inv_l,
+                                                oacc[b][dt][4 * g + 2] * inv_l, oacc[b][dt][4 * g + 3] * inv_l);
                     *reinterpret_cast<float4*>(orow + dt * 32 + 8 * g + 4 * half) = v;
                 }
             if (L && half == 0) L[(size_t)zh * N + q[b]] = row_ok ? m_run[b] + __logf(l_tot) : -INFINITY;

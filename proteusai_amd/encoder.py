@@ -1,0 +1,96 @@
+"""Encoder stack around the two kernels (inference forward).
+
+Follows the legacy transformer architecture the reference's README describes
+(README.md:38,48) and its code:
+  MLP                          utils/model_utils/base_modules/base_modules.py:6-52
+  Encoder (post-LN layer)      old/old_scripts/encoder.py:8-41
+  GeoAttention                 old/old_scripts/encoder.py:43-121  (proteusai_amd.geometric_attn.GeoAttention)
+The wavefunction embedding is added to an amino-acid embedding table and the
+sum runs through the encoder layers and a linear head to 20 amino-acid logits.
+Only plain PyTorch glue lives here; the two O(N^2) operators are the HIP kernels.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .geometric_attn import GeoAttention
+from .wf_embedding import WaveFunctionEmbedding
+
+
+class MLP(nn.Module):
+    """in_proj -> act -> [hidden -> act]* -> out_proj, dropout after each activation (base_modules.py:6-52)."""
+
+    def __init__(self, d_in=512, d_out=512, d_hidden=1024, hidden_layers=0, dropout=0.1, act="gelu"):
+        super().__init__()
+        self.in_proj = nn.Linear(d_in, d_hidden)
+        self.hidden_proj = nn.ModuleList([nn.Linear(d_hidden, d_hidden) for _ in range(hidden_layers)])
+        self.out_proj = nn.Linear(d_hidden, d_out)
+        self.in_dropout = nn.Dropout(dropout)
+        self.hidden_dropout = nn.ModuleList([nn.Dropout(dropout) for _ in range(hidden_layers)])
+        self.act = {"gelu": F.gelu, "silu": F.silu, "relu": F.relu, "sigmoid": torch.sigmoid}.get(act, lambda x: x)
+        nn.init.xavier_uniform_(self.in_proj.weight)
+        nn.init.zeros_(self.in_proj.bias)
+        for layer in self.hidden_proj:
+            nn.init.kaiming_uniform_(layer.weight, nonlinearity="relu")
+            nn.init.zeros_(layer.bias)
+        nn.init.xavier_uniform_(self.out_proj.weight)
+        nn.init.zeros_(self.out_proj.bias)
+
+    def forward(self, x):
+        x = self.in_dropout(self.act(self.in_proj(x)))
+        for hidden, dropout in zip(self.hidden_proj, self.hidden_dropout):
+            x = dropout(self.act(hidden(x)))
+        return self.out_proj(x)
+
+
+class Encoder(nn.Module):
+    """Post-LN encoder layer: LN(q + attn(q,k,v)), LN(q + ffn(q)) (old/old_scripts/encoder.py:33-41), with the
+    geometric attention branch (`bias=True, personal=False` in the reference's constructor)."""
+
+    def __init__(self, d_model=512, heads=8, d_hidden=2048, hidden_layers=0, dropout=0.10, min_spread=2.0, learn_spreads=True):
+        super().__init__()
+        self.attn = GeoAttention(d_model=d_model, heads=heads, min_spread=min_spread, learn_spreads=learn_spreads)
+        self.attn_norm = nn.LayerNorm(d_model)
+        self.ffn = MLP(d_in=d_model, d_out=d_model, d_hidden=d_hidden, hidden_layers=hidden_layers, dropout=dropout)
+        self.ffn_norm = nn.LayerNorm(d_model)
+        self.dropout = nn.Dropout(dropout)
+
+    def forward(self, q, k, v, coords, mask=None):
+        q = self.attn_norm(q + self.dropout(self.attn(q, k, v, coords, mask=mask)))
+        q = self.ffn_norm(q + self.dropout(self.ffn(q)))
+        return q
+
+
+class ProteusEncoder(nn.Module):
+    """WE(coords) + Embedding[tokens] -> `layers` encoder layers -> Linear(d_model, 20).
+
+    sigma per head is log-spaced from `sigma_min` to `sigma_max` at initialisation
+    (sigma = min_spread + exp(w), old/old_scripts/encoder.py:88-89).  The embedding runs in
+    fp32; the encoder layers run in the dtype of their weights (e.g. after `.to(torch.bfloat16)`
+    applied to `layers`, `aa_embedding` and `head`).
+    """
+
+    def __init__(self, d_model=512, heads=8, layers=4, d_hidden=2048, vocab=33, n_out=20,
+                 min_wl=3.7, max_wl=20.0, base_wl=20.0, sigma_min=3.0, sigma_max=25.0, min_spread=2.0, dropout=0.0):
+        super().__init__()
+        self.wf_embedding = WaveFunctionEmbedding(d_wf=d_model, min_wl=min_wl, max_wl=max_wl, base_wl=base_wl, anisotropic=False)
+        self.aa_embedding = nn.Embedding(vocab, d_model)
+        self.layers = nn.ModuleList([Encoder(d_model=d_model, heads=heads, d_hidden=d_hidden, dropout=dropout, min_spread=min_spread)
+                                     for _ in range(layers)])
+        self.head = nn.Linear(d_model, n_out)
+        if heads > 1:
+            sig = sigma_min * (sigma_max / sigma_min) ** (torch.arange(heads, dtype=torch.float64) / (heads - 1))
+        else:
+            sig = torch.tensor([sigma_min], dtype=torch.float64)
+        w = torch.log(sig - min_spread).to(torch.float32)
+        with torch.no_grad():
+            for layer in self.layers:
+                layer.attn.spread_weights.copy_(w)
+
+    def forward(self, coords, tokens, key_padding_mask=None):
+        wf = self.wf_embedding(coords, None, key_padding_mask=key_padding_mask)           # fp32 [Z,N,d_model]
+        x = wf + self.aa_embedding(tokens).to(wf.dtype)
+        x = x.to(self.head.weight.dtype)
+        for layer in self.layers:
+            x = layer(x, x, x, coords, mask=key_padding_mask)
+        return self.head(x)
