@@ -58,6 +58,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-attn", action="store_true", help="skip the geometric attention leg")
+    ap.add_argument("--no-encoder", action="store_true", help="skip the encoder-forward leg (BASELINE.json configs[3])")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--we-tuning", type=int, default=0)
     ap.add_argument("--copy-calib", action="store_true",
@@ -171,6 +172,35 @@ def main():
             "ms": a_ms, "tflops": a_tflops, "dtype": "bf16",
             "roofline": {"kernel": "geo_attn_fwd_kernel", "bound": "mfma", "achieved": a_tflops, "peak": PEAK_BF16_MFMA_TFLOPS,
                          "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES},
+        }
+
+    # ---------------- encoder forward, B=8, N=1024, 4 layers, bf16 weights, fp32 WE (configs[3]) ----------------
+    if not args.no_encoder:
+        import proteusai_amd as pa
+        torch.manual_seed(4)
+        model = pa.ProteusEncoder().eval().to(dev)
+        model.aa_embedding.to(torch.bfloat16)
+        model.layers.to(torch.bfloat16)
+        model.head.to(torch.bfloat16)
+        g = torch.Generator().manual_seed(4)
+        ecoords = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)]).to(dev)
+        etokens = torch.randint(0, 33, (8, 1024), generator=g).to(dev)
+        lens = torch.randint(128, 1025, (8,), generator=g)
+        emask = (torch.arange(1024)[None, :] >= lens[:, None]).to(dev)
+        with torch.no_grad():
+            for _ in range(3):
+                model(ecoords, etokens, emask)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                model(ecoords, etokens, emask)
+            e1.record()
+            torch.cuda.synchronize()
+        result["encoder_forward"] = {
+            "workload": "WE + 33x512 embedding, 4 x (geometric MHA H=8 + LN + FFN 512-2048-512 GELU + LN), head to 20; "
+                        "B=8 N=1024 lengths 128-1024, bf16 weights, fp32 WE (BASELINE.json configs[3])",
+            "ms": e0.elapsed_time(e1) / 10, "valid_tokens": int(lens.sum()),
         }
 
     # ---------------- CPU baseline: the tiled CPU PyTorch path on a bounded sample of observer rows ----------------

@@ -181,8 +181,9 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // first and last unpadded query of the workgroup (wave-level reduction, then one LDS atomic each)
     int wave_first, wave_last;
     {
-        int lo = q_ok[0] ? q[0] : (q_ok[1] ? q[1] : 0x7fffffff);
-        int hi = q_ok[1] ? q[1] : (q_ok[0] ? q[0] : -1);
+        int lo = 0x7fffffff, hi = -1;
+#pragma unroll
+        for (int b = 0; b < GA_QB; ++b) if (q_ok[b]) { lo = min(lo, q[b]); hi = max(hi, q[b]); }
         for (int o = 32; o > 0; o >>= 1) { lo = min(lo, __shfl_xor(lo, o)); hi = max(hi, __shfl_xor(hi, o)); }
         if (lane == 0) { atomicMin(&sm.q_first, lo); atomicMax(&sm.q_last, hi); }
         wave_first = lo; wave_last = hi;
@@ -218,7 +219,12 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         qx[b] = (cz[3 * qc] - ox) * cscale; qy[b] = (cz[3 * qc + 1] - oy) * cscale; qz[b] = (cz[3 * qc + 2] - oz) * cscale;
         qn2[b] = qx[b] * qx[b] + qy[b] * qy[b] + qz[b] * qz[b];
     }
-    atomicMax(&sm.rho2_bits, __builtin_bit_cast(unsigned, fmaxf(qn2[0], qn2[1])));
+    {
+        float qn2max = 0.f;
+#pragma unroll
+        for (int b = 0; b < GA_QB; ++b) qn2max = fmaxf(qn2max, qn2[b]);
+        atomicMax(&sm.rho2_bits, __builtin_bit_cast(unsigned, qn2max));
+    }
 
     // ---- sphere around this wave's queries, for the far-tile test ----
     {
@@ -512,7 +518,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
         for (int b = 0; b < GA_QB; ++b) {
             uint4 pb[2];
-            floatx16 dacc;
+            floatx16 dacc = {};
             if (near && use_mfma_dist) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) dacc[r] = 0.f;

@@ -45,17 +45,17 @@ __device__ __forceinline__ float sgpr(float v) {
 // FRACT: reduce the phase to [0,1) revolutions before v_sin/v_cos (needed only when it can exceed
 // the +-256 revolutions those instructions accept).
 template <int KT, bool FRACT>
-__device__ __forceinline__ void stream_sources(const float4* s_keys, const int nk,
+__device__ __forceinline__ void stream_sources(const float4* s_keys, const int first, const int step, const int nk,
                                                const float xi, const float yi, const float zi,
                                                const float (&kr)[KT],
                                                float (&acc_oc)[KT], float (&acc_os)[KT],
                                                float (&acc_c)[KT], float (&acc_s)[KT], float& nzero)
 {
-    float4 knext = s_keys[0];
+    float4 knext = s_keys[first];                 // (reads at most WE_WAVES entries past nk: the array is padded)
 #pragma unroll 1
-    for (int jj = 0; jj < nk; ++jj) {
+    for (int jj = first; jj < nk; jj += step) {
         const float4 kj = knext;
-        knext = s_keys[jj + 1];
+        knext = s_keys[jj + step];
         const float dx = xi - kj.x, dy = yi - kj.y, dz = zi - kj.z;
         const float r2 = dx * dx + dy * dy + dz * dz;
         const bool  ok = r2 != 0.0f;
@@ -79,32 +79,143 @@ __device__ __forceinline__ void stream_sources(const float4* s_keys, const int n
     }
 }
 
-// KT     wavenumbers per wave (4*KT accumulators per lane)
-// SPLIT  the sources are split over gridDim.x/ceil(N/64) workgroups and partial
-//        sums are added to pre-zeroed outputs with float atomics (small N only)
-// FRACT  this instantiation reduces the phase explicitly.  Both instantiations are launched over the
-//        same grid; a workgroup runs in the FRACT=false kernel if no phase of its waves can leave
-//        +-WE_MAX_REV revolutions and in the FRACT=true kernel otherwise (it returns at once from
-//        the other one), unless take_all forces one kernel to take every workgroup.
+// Everything after the prologue, for one choice of FRACT: the running sums live only inside this
+// function, so the two instantiations a kernel holds never have their accumulators alive together.
 template <int KT, bool SPLIT, bool FRACT>
+__device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_red,
+                                        const float* __restrict__ cz, const uint8_t* __restrict__ mz, const int layout,
+                                        float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
+                                        const int N, const int K, const size_t zN,
+                                        const int tid, const int lane, const int wave,
+                                        const int i, const bool i_in, const bool i_valid, const bool any_valid,
+                                        const float xi, const float yi, const float zi,
+                                        const int k0, const bool wave_active, const float (&kr)[KT])
+{
+    float acc_oc[KT], acc_os[KT], acc_c[KT], acc_s[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) { acc_oc[t] = 0.f; acc_os[t] = 0.f; acc_c[t] = 0.f; acc_s[t] = 0.f; }
+    float nzero = 0.f;
+
+    if (any_valid) {
+        const int j_end = N;
+        for (int jb = 0; jb < j_end; jb += WE_JB) {
+            // -- stage one block of sources, keeping only the unpadded ones --
+            const int  j    = jb + tid;
+            const bool j_in = j < j_end;
+            const int  jc   = j_in ? j : N - 1;
+            float xj, yj, zj;
+            if (layout == PROTEUS_COORDS_SOA) { xj = cz[jc]; yj = cz[(size_t)N + jc]; zj = cz[2 * (size_t)N + jc]; }
+            else                              { xj = cz[3 * (size_t)jc]; yj = cz[3 * (size_t)jc + 1]; zj = cz[3 * (size_t)jc + 2]; }
+            const bool j_valid = j_in && !(mz && mz[jc]);
+
+            const uint64_t bal   = __builtin_amdgcn_ballot_w64(j_valid);
+            const int      below = __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+            __syncthreads();                       // previous block fully consumed
+            if (lane == 0) s_wcount[wave] = __builtin_popcountll(bal);
+            __syncthreads();
+            int base = 0, nk = 0;
+#pragma unroll
+            for (int w = 0; w < WE_WAVES; ++w) { const int c = s_wcount[w]; base += (w < wave) ? c : 0; nk += c; }
+            if (j_valid) s_keys[base + below] = make_float4(xj, yj, zj, 0.f);
+            __syncthreads();
+            nk = __builtin_amdgcn_readfirstlane(nk);
+
+            if (!wave_active) continue;
+
+            // -- stream the staged sources --
+            if (SPLIT) stream_sources<KT, FRACT>(s_keys, wave, WE_WAVES, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
+            else       stream_sources<KT, FRACT>(s_keys, 0, 1, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
+        }
+    }
+
+    if (SPLIT) {
+        // ---- the four waves' partial sums meet in LDS; wave 0 writes the rows ----
+        __syncthreads();
+        if (wave > 0) {
+            float* r = s_red + (size_t)(wave - 1) * (4 * KT + 1) * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+                r[(4 * t + 0) * 64] = acc_oc[t]; r[(4 * t + 1) * 64] = acc_os[t];
+                r[(4 * t + 2) * 64] = acc_c[t];  r[(4 * t + 3) * 64] = acc_s[t];
+            }
+            r[4 * KT * 64] = nzero;
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < WE_WAVES - 1; ++w) {
+            const float* r = s_red + (size_t)w * (4 * KT + 1) * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+                acc_oc[t] += r[(4 * t + 0) * 64]; acc_os[t] += r[(4 * t + 1) * 64];
+                acc_c[t]  += r[(4 * t + 2) * 64]; acc_s[t]  += r[(4 * t + 3) * 64];
+            }
+            nzero += r[4 * KT * 64];
+        }
+    }
+
+    if (!wave_active || !i_in) return;
+
+    // ---- epilogue: each lane writes its own rows ----
+    const size_t row = zN + (size_t)i;
+    float* o  = out      + row * (size_t)(2 * K) + 2 * (size_t)k0;
+    float* pc = cos_sums + row * (size_t)K + k0;
+    float* ps = sin_sums + row * (size_t)K + k0;
+
+    const float keep = i_valid ? 1.0f : 0.0f;    // padded observer: zeros
+    if (k0 + KT <= K && (K & 1) == 0 && (KT & 3) == 0 && (K & 3) == 0) {
+        // full tile, rows 16-byte aligned: vector stores
+#pragma unroll
+        for (int t = 0; t < KT; t += 2) {
+            float4 v = make_float4(acc_oc[t] * keep, acc_os[t] * keep, acc_oc[t + 1] * keep, acc_os[t + 1] * keep);
+            *reinterpret_cast<float4*>(o + 2 * t) = v;
+        }
+#pragma unroll
+        for (int t = 0; t < KT; t += 4) {
+            float4 c = make_float4((acc_c[t] - nzero) * keep, (acc_c[t + 1] - nzero) * keep,
+                                   (acc_c[t + 2] - nzero) * keep, (acc_c[t + 3] - nzero) * keep);
+            float4 s = make_float4(acc_s[t] * keep, acc_s[t + 1] * keep, acc_s[t + 2] * keep, acc_s[t + 3] * keep);
+            *reinterpret_cast<float4*>(pc + t) = c;
+            *reinterpret_cast<float4*>(ps + t) = s;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            if (k0 + t < K) {
+                o[2 * t]     = acc_oc[t] * keep;
+                o[2 * t + 1] = acc_os[t] * keep;
+                pc[t] = (acc_c[t] - nzero) * keep;
+                ps[t] = acc_s[t] * keep;
+            }
+        }
+    }
+}
+
+// KT     wavenumbers per wave (4*KT accumulators per lane)
+// SPLIT  small problems: the four waves of a workgroup share ONE wavenumber tile and split the staged
+//        sources between them (wave w takes sources w, w+4, ...); the partial sums meet in LDS at the
+//        end.  Four times as many workgroups for the same KT, still no atomics, still deterministic.
+// fract_mode  0: a workgroup reduces the phase explicitly (v_fract) only if some phase of its waves can
+//        leave +-WE_MAX_REV revolutions; 1: always; -1: never (a measuring aid, valid only for bounded phases)
+template <int KT, bool SPLIT>
 __global__ __launch_bounds__(WE_THREADS)
 void we_fwd_kernel(const float* __restrict__ coords, const int layout,
                    const float* __restrict__ wavenumbers,
                    const uint8_t* __restrict__ mask,
                    float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
-                   const int N, const int K, const int nsplit, const int take_all)
+                   const int N, const int K, const int fract_mode)
 {
-    __shared__ float4 s_keys[WE_JB + 1];   // +1: the stream loop reads one source ahead
+    __shared__ float4 s_keys[WE_JB + WE_WAVES];   // padding: the stream loop reads one step ahead
     __shared__ int    s_wcount[WE_WAVES];
     __shared__ float  s_box[WE_WAVES][6];
+    __shared__ float  s_red[SPLIT ? (WE_WAVES - 1) * (4 * KT + 1) * 64 : 1];
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int z    = blockIdx.z;
 
-    int iblock = blockIdx.x, split = 0;
-    if (SPLIT) { iblock = blockIdx.x / nsplit; split = blockIdx.x - iblock * nsplit; }
+    const int iblock = blockIdx.x;
 
     const size_t zN = (size_t)z * (size_t)N;
     const float* cz = coords + zN * 3;
@@ -124,7 +235,7 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     const bool any_valid = __builtin_amdgcn_ballot_w64(i_valid) != 0;
 
     // ---- this wave's wavenumbers, converted to revolutions per angstrom ----
-    const int  k0          = (blockIdx.y * WE_WAVES + wave) * KT;
+    const int  k0          = SPLIT ? blockIdx.y * KT : (blockIdx.y * WE_WAVES + wave) * KT;
     const bool wave_active = k0 < K;
     float kr[KT];
 #pragma unroll
@@ -138,6 +249,7 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     for (int t = 0; t < KT; ++t) kr_max = fmaxf(kr_max, fabsf(kr[t]));
 
     // ---- can any phase of this wave leave the +-256 revolutions v_sin/v_cos accept? ----
+    bool wg_safe = false;
     // Bounding box of all coordinates of the batch item (a few loads per thread, once), then the
     // distance from each observer to its farthest corner bounds every r_ij of the lane.
     {
@@ -170,122 +282,20 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
         const bool wave_safe = __builtin_amdgcn_ballot_w64(!(rfar * kr_max < WE_MAX_REV)) == 0;
         if (lane == 0) s_wcount[wave] = wave_safe ? 1 : 0;
         __syncthreads();
-        const bool wg_safe = (s_wcount[0] & s_wcount[1] & s_wcount[2] & s_wcount[3]) != 0;
-        if (!take_all && wg_safe == FRACT) return;      // the other instantiation owns this workgroup
+        wg_safe = (s_wcount[0] & s_wcount[1] & s_wcount[2] & s_wcount[3]) != 0;
     }
-
-    float acc_oc[KT], acc_os[KT], acc_c[KT], acc_s[KT];
-#pragma unroll
-    for (int t = 0; t < KT; ++t) { acc_oc[t] = 0.f; acc_os[t] = 0.f; acc_c[t] = 0.f; acc_s[t] = 0.f; }
-    float nzero = 0.f;
-
-    if (any_valid) {
-        // sources handled by this workgroup
-        int j_begin = 0, j_end = N;
-        if (SPLIT) {
-            const int chunk = ((N + nsplit - 1) / nsplit + WE_JB - 1) / WE_JB * WE_JB;
-            j_begin = split * chunk;
-            j_end   = min(N, j_begin + chunk);
-        }
-
-        for (int jb = j_begin; jb < j_end; jb += WE_JB) {
-            // -- stage one block of sources, keeping only the unpadded ones --
-            const int  j    = jb + tid;
-            const bool j_in = j < j_end;
-            const int  jc   = j_in ? j : N - 1;
-            float xj, yj, zj;
-            if (layout == PROTEUS_COORDS_SOA) { xj = cz[jc]; yj = cz[(size_t)N + jc]; zj = cz[2 * (size_t)N + jc]; }
-            else                              { xj = cz[3 * (size_t)jc]; yj = cz[3 * (size_t)jc + 1]; zj = cz[3 * (size_t)jc + 2]; }
-            const bool j_valid = j_in && !(mz && mz[jc]);
-
-            const uint64_t bal   = __builtin_amdgcn_ballot_w64(j_valid);
-            const int      below = __builtin_popcountll(bal & ((1ull << lane) - 1ull));
-            __syncthreads();                       // previous block fully consumed
-            if (lane == 0) s_wcount[wave] = __builtin_popcountll(bal);
-            __syncthreads();
-            int base = 0, nk = 0;
-#pragma unroll
-            for (int w = 0; w < WE_WAVES; ++w) { const int c = s_wcount[w]; base += (w < wave) ? c : 0; nk += c; }
-            if (j_valid) s_keys[base + below] = make_float4(xj, yj, zj, 0.f);
-            __syncthreads();
-            nk = __builtin_amdgcn_readfirstlane(nk);
-
-            if (!wave_active) continue;
-
-            // -- stream the staged sources --
-            stream_sources<KT, FRACT>(s_keys, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
-        }
-    }
-
-    if (!wave_active || !i_in) return;
-
-    // ---- epilogue: each lane writes its own rows ----
-    const size_t row = zN + (size_t)i;
-    float* o  = out      + row * (size_t)(2 * K) + 2 * (size_t)k0;
-    float* pc = cos_sums + row * (size_t)K + k0;
-    float* ps = sin_sums + row * (size_t)K + k0;
-
-    if (SPLIT) {
-        if (!i_valid) return;                    // outputs were pre-zeroed
-#pragma unroll
-        for (int t = 0; t < KT; ++t) {
-            if (k0 + t < K) {
-                unsafeAtomicAdd(o + 2 * t,     acc_oc[t]);
-                unsafeAtomicAdd(o + 2 * t + 1, acc_os[t]);
-                unsafeAtomicAdd(pc + t, acc_c[t] - nzero);
-                unsafeAtomicAdd(ps + t, acc_s[t]);
-            }
-        }
-        return;
-    }
-
-    const float keep = i_valid ? 1.0f : 0.0f;    // padded observer: zeros
-    if (k0 + KT <= K && (K & 1) == 0 && (KT & 3) == 0 && (K & 3) == 0) {
-        // full tile, rows 16-byte aligned: vector stores
-#pragma unroll
-        for (int t = 0; t < KT; t += 2) {
-            float4 v = make_float4(acc_oc[t] * keep, acc_os[t] * keep, acc_oc[t + 1] * keep, acc_os[t + 1] * keep);
-            *reinterpret_cast<float4*>(o + 2 * t) = v;
-        }
-#pragma unroll
-        for (int t = 0; t < KT; t += 4) {
-            float4 c = make_float4((acc_c[t] - nzero) * keep, (acc_c[t + 1] - nzero) * keep,
-                                   (acc_c[t + 2] - nzero) * keep, (acc_c[t + 3] - nzero) * keep);
-            float4 s = make_float4(acc_s[t] * keep, acc_s[t + 1] * keep, acc_s[t + 2] * keep, acc_s[t + 3] * keep);
-            *reinterpret_cast<float4*>(pc + t) = c;
-            *reinterpret_cast<float4*>(ps + t) = s;
-        }
-    } else {
-#pragma unroll
-        for (int t = 0; t < KT; ++t) {
-            if (k0 + t < K) {
-                o[2 * t]     = acc_oc[t] * keep;
-                o[2 * t + 1] = acc_os[t] * keep;
-                pc[t] = (acc_c[t] - nzero) * keep;
-                ps[t] = acc_s[t] * keep;
-            }
-        }
-    }
+    const bool use_fract = fract_mode > 0 || (fract_mode == 0 && !wg_safe);
+    if (use_fract)
+        we_body<KT, SPLIT, true>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
+                                 i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
+    else
+        we_body<KT, SPLIT, false>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
+                                  i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
 }
 
-__global__ void we_zero_kernel(float4* p, size_t n4, float* tail, int ntail) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n4; idx += stride)
-        p[idx] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (blockIdx.x == 0 && (int)threadIdx.x < ntail) tail[threadIdx.x] = 0.f;
-}
 
-void zero_async(float* p, size_t n, hipStream_t st) {
-    // a plain fill kernel rather than a memset node, so callers may capture it
-    const size_t n4 = n / 4;
-    const int ntail = (int)(n - n4 * 4);
-    const int blocks = (int)((n4 + 255) / 256 > 4096 ? 4096 : ((n4 + 255) / 256 ? (n4 + 255) / 256 : 1));
-    hipLaunchKernelGGL(we_zero_kernel, dim3(blocks), dim3(256), 0, st,
-                       reinterpret_cast<float4*>(p), n4, p + n4 * 4, ntail);
-}
-
-// fract: 0 = each workgroup picks (two cooperating launches), 1 = always reduce, -1 = never reduce
-// (only valid when every phase is known to stay within +-256 revolutions; a measuring aid)
+// fract: 0 = each workgroup picks, 1 = always reduce, -1 = never reduce (only valid when every phase
+// is known to stay within +-256 revolutions; a measuring aid)
 struct WeVariant { const char* name; int kt; bool split; int fract; };
 // index 0 is "automatic"; the others force a tile
 const WeVariant kVariants[] = {
@@ -293,8 +303,6 @@ const WeVariant kVariants[] = {
     {"kt32", 32, false, 0},
     {"kt16", 16, false, 0},
     {"kt8", 8, false, 0},
-    {"kt64", 64, false, 0},
-    {"kt32_split", 32, true, 0},
     {"kt16_split", 16, true, 0},
     {"kt8_split", 8, true, 0},
     {"kt32_fract", 32, false, 1},
@@ -304,22 +312,13 @@ constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 template <int KT, bool SPLIT>
 int launch(const float* coords, int layout, const float* wn, const uint8_t* mask,
-           float* out, float* cs, float* ss, int Z, int N, int K, int nsplit, int fract, hipStream_t st)
+           float* out, float* cs, float* ss, int Z, int N, int K, int fract, hipStream_t st)
 {
     const int iblocks = (N + 63) / 64;
-    const int ktiles  = (K + KT * WE_WAVES - 1) / (KT * WE_WAVES);
-    if (SPLIT) {
-        zero_async(out, (size_t)Z * N * 2 * K, st);
-        zero_async(cs,  (size_t)Z * N * K, st);
-        zero_async(ss,  (size_t)Z * N * K, st);
-    }
-    dim3 grid(iblocks * (SPLIT ? nsplit : 1), ktiles, Z);
-    if (fract <= 0)
-        hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT, false>), grid, dim3(WE_THREADS), 0, st,
-                           coords, layout, wn, mask, out, cs, ss, N, K, nsplit, fract < 0 ? 1 : 0);
-    if (fract >= 0)
-        hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT, true>), grid, dim3(WE_THREADS), 0, st,
-                           coords, layout, wn, mask, out, cs, ss, N, K, nsplit, fract > 0 ? 1 : 0);
+    const int ktiles  = SPLIT ? (K + KT - 1) / KT : (K + KT * WE_WAVES - 1) / (KT * WE_WAVES);
+    dim3 grid(iblocks, ktiles, Z);
+    hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT>), grid, dim3(WE_THREADS), 0, st,
+                       coords, layout, wn, mask, out, cs, ss, N, K, fract);
     return (int)hipGetLastError();
 }
 
@@ -360,27 +359,30 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
     const int fract = kVariants[tuning].fract;
     const long iblocks = ((long)N + 63) / 64 * Z;
     if (tuning == 0) {
-        // Aim for at least two waves on each of the 1024 SIMDs; prefer the
-        // widest wavenumber tile (least per-pair overhead) that achieves it.
-        const long want = 2048;
-        kt = 32;
-        while (kt > 8 && iblocks * ((K + kt - 1) / kt) < want) kt >>= 1;
-        if (kt > K) { kt = 8; while (kt < K && kt < 32) kt <<= 1; }
-        split = iblocks * ((K + kt - 1) / kt) < want / 2 && N >= 2 * WE_JB;
+        // Pick the (wavenumber tile, source split) pair with the least estimated issue time:
+        // instructions per wave x rounds of 1024 waves, with a penalty when a SIMD would hold a
+        // single wave (nothing to cover its LDS and transcendental latencies).  Ties keep the
+        // earlier candidate (wider tile, no split).
+        static const int cand_kt[5]    = {32, 16, 8, 16, 8};
+        static const int cand_split[5] = {0, 0, 0, 1, 1};
+        double best = 1e300;
+        for (int c = 0; c < 5; ++c) {
+            const int  ckt = cand_kt[c];
+            const bool csp = cand_split[c] != 0;
+            if (csp && N < 4 * 64) continue;
+            const long ktiles = ((long)K + ckt - 1) / ckt;
+            const long nwaves = csp ? iblocks * ktiles * WE_WAVES : iblocks * ((ktiles + WE_WAVES - 1) / WE_WAVES) * WE_WAVES;
+            const double keys = csp ? (double)N / WE_WAVES : (double)N;
+            const double rounds = (double)((nwaves + 1023) / 1024);
+            double est = rounds * keys * (8.0 * ckt + 17.0);
+            if (nwaves < 2048) est *= 1.25;
+            if (est < best * 0.999) { best = est; kt = ckt; split = csp; }
+        }
     }
-    int nsplit = 1;
-    if (split) {
-        const long waves = iblocks * ((K + kt - 1) / kt);
-        nsplit = (int)((2048 + waves - 1) / waves);
-        const int maxsplit = (N + WE_JB - 1) / WE_JB;
-        if (nsplit > maxsplit) nsplit = maxsplit;
-        if (nsplit < 1) nsplit = 1;
-    }
-#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, nsplit, fract, st) \
-                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, fract, st))
+#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st) \
+                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st))
     switch (kt) {
-        case 64: return launch<64, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 1, fract, st);
-        case 32: return WE_GO(32);
+        case 32: return launch<32, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st);
         case 16: return WE_GO(16);
         default: return WE_GO(8);
     }
