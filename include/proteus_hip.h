@@ -129,6 +129,23 @@ int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint1
                                const float* O, const float* L,
                                int Z, int H, int N, int d_head, int tuning);
 
+/*
+ * The same kernel with the logits of the reference's Triton kernel instead of
+ * the README multiplier (old/old_scripts/attn/geometric_attn.py:193-201, launch
+ * :588-599; dense statement tests/attn/geo_attn.py:194-210):
+ *     rbf   = exp(-|r_i - r_j|^2 / (2 sigma_h^2))
+ *     s_ij  = S_ij + beta_h * (2 (rbf - min_rbf)/(max_rbf - min_rbf) - 1) * |S_ij|,   S_ij = q_i.k_j/sqrt(d)
+ *     s_ij  = -inf where key j or query i is padded or rbf is outside [min_rbf, max_rbf]
+ *   beta [H] f32; requires max_rbf > min_rbf.  Everything else as proteus_geo_attn_fwd
+ *   (operands are bf16 here, fp16 in the reference).
+ */
+int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                const float* coords, const float* sigma, const float* beta,
+                                const uint8_t* key_pad_mask,
+                                float* O, float* L,
+                                int Z, int H, int N, int d_head,
+                                float min_rbf, float max_rbf, int tuning, void* stream);
+
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);
 

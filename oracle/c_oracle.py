@@ -87,3 +87,28 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, rows=None):
        ctypes.c_int(Z), ctypes.c_int(H), ctypes.c_int(N), ctypes.c_int(d),
        _p(r, ctypes.c_int), ctypes.c_int(R), _p(O, ctypes.c_double), _p(L, ctypes.c_double))
     return O, L
+
+
+def geo_attn_legacy(Q, K, V, coords, sigma, beta, key_padding_mask=None, min_rbf=0.0, max_rbf=1.0, rows=None):
+    """The reference kernel's own logits, S + beta*rbf_norm*|S| with the [min_rbf, max_rbf] pair mask.
+    Same conventions as geo_attn.  Returns (O, L) in float64."""
+    q = np.ascontiguousarray(np.asarray(Q, dtype=np.float32))
+    k = np.ascontiguousarray(np.asarray(K, dtype=np.float32))
+    v = np.ascontiguousarray(np.asarray(V, dtype=np.float32))
+    c = np.ascontiguousarray(np.asarray(coords, dtype=np.float32))
+    s = np.ascontiguousarray(np.asarray(sigma, dtype=np.float32))
+    b = np.ascontiguousarray(np.asarray(beta, dtype=np.float32))
+    Z, H, N, d = q.shape
+    assert k.shape == q.shape and v.shape == q.shape and c.shape == (Z, N, 3) and s.shape == (H,) and b.shape == (H,)
+    m = None if key_padding_mask is None else np.ascontiguousarray(np.asarray(key_padding_mask).astype(np.uint8))
+    r, R = _rows(rows, N)
+    O = np.empty((Z, H, R, d), np.float64)
+    L = np.empty((Z, H, R), np.float64)
+    fn = lib().geo_attn_legacy_oracle_f64
+    fn.restype = None
+    fn(_p(q, ctypes.c_float), _p(k, ctypes.c_float), _p(v, ctypes.c_float), _p(c, ctypes.c_float),
+       _p(s, ctypes.c_float), _p(b, ctypes.c_float), _p(m, ctypes.c_uint8),
+       ctypes.c_int(Z), ctypes.c_int(H), ctypes.c_int(N), ctypes.c_int(d),
+       ctypes.c_double(min_rbf), ctypes.c_double(max_rbf),
+       _p(r, ctypes.c_int), ctypes.c_int(R), _p(O, ctypes.c_double), _p(L, ctypes.c_double))
+    return O, L

@@ -101,3 +101,24 @@ def geo_attn_torch(Q, K, V, coords, sigma, key_padding_mask=None, rows=None, row
             O[z][:, a:a + idx.numel()] = torch.matmul(P, V[z])
             L[z][:, a:a + idx.numel()] = Lz
     return O, L
+
+
+def geo_attn_legacy_torch(Q, K, V, coords, spreads, b, mask=None, min_rbf=0.0, max_rbf=1.0, dtype=torch.float32):
+    """The reference's dense statement of its own kernel, line for line in meaning
+    (tests/attn/geo_attn.py:172-212, torch_attn): S = QK^T/sqrt(d); dists; rbfs = exp(-dists^2/(2 spreads^2));
+    attn_mask = mask_i | mask_j | rbfs < min_rbf | rbfs > max_rbf; rbfs = 2(rbfs-min)/(max-min) - 1;
+    S = where(attn_mask, -inf, S + b*rbfs*|S|); softmax; P V.  Fully masked rows are returned as zeros
+    (the kernel's convention, old/old_scripts/attn/geometric_attn.py:233) instead of NaN."""
+    Q, K, V = Q.to(dtype), K.to(dtype), V.to(dtype)
+    coords, spreads, b = coords.to(dtype), spreads.to(dtype), b.to(dtype)
+    Z, H, N, d = Q.shape
+    mask = torch.zeros(Z, N, dtype=torch.bool) if mask is None else mask.bool()
+    S = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(d)
+    dists = torch.sqrt(torch.sum((coords[:, :, None, :] - coords[:, None, :, :]) ** 2, dim=3))[:, None, :, :]
+    rbfs = torch.exp(-(dists ** 2) / (2 * (spreads[None, :, None, None] ** 2)))
+    attn_mask = mask[:, None, :, None] | mask[:, None, None, :] | (rbfs < min_rbf) | (rbfs > max_rbf)
+    rbfs = (2 * (rbfs - min_rbf) / (max_rbf - min_rbf)) - 1
+    S = torch.where(attn_mask, torch.full_like(S, float("-inf")), S + b[None, :, None, None] * rbfs * torch.abs(S))
+    P = torch.softmax(S, dim=-1)
+    P = torch.where(torch.isnan(P), torch.zeros_like(P), P)
+    return torch.matmul(P, V), torch.logsumexp(S, dim=-1)

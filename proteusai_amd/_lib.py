@@ -16,7 +16,7 @@ COORDS_AOS = 1
 SYMBOLS = [
     "proteus_version", "proteus_strerror",
     "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_num_variants", "proteus_we_variant_name",
-    "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_num_variants",
+    "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_probe_valu_rate", "proteus_probe_sincos",
 ]
@@ -51,6 +51,9 @@ def load():
     lib.proteus_we_variant_name.argtypes = [ci]
     lib.proteus_geo_attn_fwd.restype = ci
     lib.proteus_geo_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.proteus_geo_attn_legacy_fwd.restype = ci
+    lib.proteus_geo_attn_legacy_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci,
+                                                ctypes.c_float, ctypes.c_float, ci, vp]
     lib.proteus_geo_attn_fwd_check.restype = ci
     lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_num_variants.restype = ci

@@ -118,13 +118,17 @@ __device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
 // the vector ALU.  Both instantiations are launched over the same grid; unless take_all is set, a
 // workgroup runs in the matrix-core kernel if its queries lie within GA_MFMA_DIST_MAX_RHO2 of their
 // origin and in the vector-ALU kernel otherwise, and returns at once from the other one.
-template <bool DIST_VALU>
+// LEGACY selects the logits of the reference's Triton kernel instead of the README multiplier:
+//   s = S + beta_h * (2 (rbf - min_rbf)/(max_rbf - min_rbf) - 1) * |S|, pairs with rbf outside [min_rbf, max_rbf] masked
+//   (old/old_scripts/attn/geometric_attn.py:193-201).
+template <bool DIST_VALU, bool LEGACY>
 __global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                          const uint16_t* __restrict__ V, const float* __restrict__ coords,
                          const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                          float* __restrict__ O, float* __restrict__ L,
-                         const int H, const int N, const int ZH, const int n_qtiles, const int take_all)
+                         const int H, const int N, const int ZH, const int n_qtiles, const int take_all,
+                         const float* __restrict__ beta, const float min_rbf, const float max_rbf)
 {
     __shared__ Smem sm;
 
@@ -165,6 +169,10 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const float sg = sigma[h];
     // exp(-d^2/(2 sg^2)) = exp2(-(d*cs)^2) with cs = sqrt(log2(e)/2)/sg
     const float cscale = 0.84932180028801907f / sg;
+    // legacy logits: beta * rbf_norm = rbf * lg_a + lg_b
+    const float lg_beta = LEGACY ? beta[h] : 0.f;
+    const float lg_a = LEGACY ? 2.0f * lg_beta / (max_rbf - min_rbf) : 0.f;
+    const float lg_b = LEGACY ? -lg_beta * (2.0f * min_rbf / (max_rbf - min_rbf) + 1.0f) : 0.f;
     if (tid == 0) { sm.n_eff = mz ? 0 : N; sm.rho2_bits = 0u; sm.q_first = 0x7fffffff; sm.q_last = -1; }
     __syncthreads();
 
@@ -419,6 +427,13 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         }
     };
 
+    auto apply_rbf = [&](const float sv, float rbf) -> float {
+        if (!LEGACY) return __builtin_fmaf(sv, rbf, sv);
+        rbf = fminf(rbf, 1.0f);          // the matrix-core distance can come out a rounding error below zero
+        const float t = __builtin_fmaf(__builtin_fmaf(rbf, lg_a, lg_b), fabsf(sv), sv);
+        return (rbf >= min_rbf && rbf <= max_rbf) ? t : -INFINITY;
+    };
+
     // multiplier, mask, online softmax of one 32-key x 32-query block; returns P^T packed for the two
     // K=16 steps.  Accumulator register r of key block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4).
     auto softmax_block = [&](const TileBuf& tb, const int mt, const int b, floatx16& sacc, const floatx16& dacc,
@@ -426,10 +441,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         if (near) {
             if (use_mfma_dist) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float rbf = __builtin_amdgcn_exp2f(dacc[r]);
-                    sacc[r] = __builtin_fmaf(sacc[r], rbf, sacc[r]);
-                }
+                for (int r = 0; r < 16; ++r) sacc[r] = apply_rbf(sacc[r], __builtin_amdgcn_exp2f(dacc[r]));
             } else {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
@@ -444,9 +456,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                     for (int v = 0; v < 4; ++v) {
                         const float dx = qx[b] - kxs[v], dy = qy[b] - kys[v], dz = qz[b] - kzs[v];
                         const float d2 = dx * dx + dy * dy + dz * dz;
-                        const float rbf = __builtin_amdgcn_exp2f(-d2);
-                        const float sv = sacc[4 * g + v];
-                        sacc[4 * g + v] = __builtin_fmaf(sv, rbf, sv);
+                        sacc[4 * g + v] = apply_rbf(sacc[4 * g + v], __builtin_amdgcn_exp2f(-d2));
                     }
                 }
             }
@@ -553,7 +563,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         const TileBuf& tb = sm.tile[t & 1];
         const bool has_valid  = tb.flags[1] != 0;
         const bool has_masked = tb.flags[0] != 0;
-        const bool near       = tb.near[wave] == t + 1;
+        const bool near       = LEGACY || tb.near[wave] == t + 1;
         if (has_valid) {
             key_block(tb, 0, has_masked, near);
             key_block(tb, 1, has_masked, near);
@@ -615,6 +625,27 @@ extern "C" int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, 
     return PROTEUS_OK;
 }
 
+namespace {
+template <bool LEGACY>
+int launch_attn(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
+                const float* beta, float min_rbf, float max_rbf, hipStream_t st)
+{
+    const int n_qtiles = (N + GA_BM - 1) / GA_BM;
+    const int ZH = Z * H;
+    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
+    // tuning 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
+    // 1 / 2: force the matrix-core / vector-ALU path everywhere
+    if (tuning != 2)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 1 ? 1 : 0, beta, min_rbf, max_rbf);
+    if (tuning != 1)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 2 ? 1 : 0, beta, min_rbf, max_rbf);
+    return (int)hipGetLastError();
+}
+}  // namespace
+
 extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                                     const float* coords, const float* sigma,
                                     const uint8_t* key_pad_mask,
@@ -623,17 +654,23 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
 {
     const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
     if (rc != PROTEUS_OK) return rc;
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const int n_qtiles = (N + GA_BM - 1) / GA_BM;
-    const int ZH = Z * H;
-    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
-    // tuning 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
-    // 1 / 2: force the matrix-core / vector-ALU path everywhere
-    if (tuning != 2)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<false>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 1 ? 1 : 0);
-    if (tuning != 1)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<true>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 2 ? 1 : 0);
-    return (int)hipGetLastError();
+    return launch_attn<false>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f,
+                              reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                           const float* coords, const float* sigma, const float* beta,
+                                           const uint8_t* key_pad_mask,
+                                           float* O, float* L,
+                                           int Z, int H, int N, int d_head,
+                                           float min_rbf, float max_rbf, int tuning, void* stream)
+{
+    const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    if (!beta) return PROTEUS_ERR_NULL_POINTER;
+    if (!(max_rbf > min_rbf)) return PROTEUS_ERR_BAD_SHAPE;
+    // a pair mask makes the result sensitive to the last bits of the rbf: use direct distances then
+    if (tuning == 0 && (min_rbf > 0.f || max_rbf < 1.f)) tuning = 2;
+    return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf,
+                             reinterpret_cast<hipStream_t>(stream));
 }

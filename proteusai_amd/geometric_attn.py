@@ -12,7 +12,8 @@ import torch.nn as nn
 from . import _lib
 
 
-def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0):
+def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0,
+             betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0):
     """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None).
 
     Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569),
@@ -20,6 +21,10 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     key_padding_mask: True = padded.  Padded query rows and rows without a
     valid key give O = 0 and logsumexp = -inf.  With return_lse the
     logsumexp L [Z,H,N] is returned as well.
+
+    With `betas` [H] the logits are those of the reference's kernel instead,
+    S + beta_h*(2(rbf-min_rbf)/(max_rbf-min_rbf)-1)*|S| with pairs whose rbf lies outside
+    [min_rbf, max_rbf] masked (old/old_scripts/attn/geometric_attn.py:193-201).
     """
     if not (Q.shape == K.shape == V.shape):
         raise AssertionError(f"Q, K, and V projection shapes must match, but got {Q.shape=}, {K.shape=}, {V.shape=}")
@@ -52,9 +57,18 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         return (O, L) if return_lse else O
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
-                                      None if m is None else m.data_ptr(),
-                                      O.data_ptr(), L.data_ptr(), Z, H, N, d, int(tuning), stream)
+        if betas is None:
+            rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
+                                          None if m is None else m.data_ptr(),
+                                          O.data_ptr(), L.data_ptr(), Z, H, N, d, int(tuning), stream)
+        else:
+            if betas.dim() != 1 or betas.size(0) != H:
+                raise AssertionError(f"number of betas must be equal to nheads, not {tuple(betas.shape)} and {H=}")
+            bt = betas.detach().to(device=dev, dtype=torch.float32).contiguous()
+            rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
+                                                 bt.data_ptr(), None if m is None else m.data_ptr(),
+                                                 O.data_ptr(), L.data_ptr(), Z, H, N, d,
+                                                 float(min_rbf), float(max_rbf), int(tuning), stream)
     _lib.check(rc, "proteus_geo_attn_fwd")
     return (O, L) if return_lse else O
 
@@ -63,8 +77,8 @@ class _geometric_attn(torch.autograd.Function):
     """Forward only: the backward kernel of the reference (geometric_attn.py:262-543) is not implemented."""
 
     @staticmethod
-    def forward(ctx, Q, K, V, coords, spreads, key_padding_mask):
-        return geo_attn(Q, K, V, coords, spreads, key_padding_mask)
+    def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf):
+        return geo_attn(Q, K, V, coords, spreads, key_padding_mask, betas=betas, min_rbf=min_rbf, max_rbf=max_rbf)
 
     @staticmethod
     def backward(ctx, dO):
@@ -74,16 +88,13 @@ class _geometric_attn(torch.autograd.Function):
 def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00):
     """Same call as the reference's geometric_attn (geometric_attn.py:545-548).
 
-    The logits are the README form S*(1+RBF); the reference kernel's
-    beta-weighted bias S + beta*RBF_norm*|S| and its [min_rbf, max_rbf] pair
-    mask are not implemented: `betas` must be None and the rbf range must be
-    the full [0, 1].
+    betas=None selects the README logits S*(1+RBF) (README.md:40; the rbf range must then be the full
+    [0, 1]); a betas tensor selects the reference kernel's own logits S + beta*RBF_norm*|S| with its
+    [min_rbf, max_rbf] pair mask (geometric_attn.py:193-201).
     """
-    if betas is not None:
-        raise NotImplementedError("the beta-weighted bias of the legacy kernel is not implemented; pass betas=None")
-    if min_rbf > 0.0 or max_rbf < 1.0:
-        raise NotImplementedError("the [min_rbf, max_rbf] pair mask is not implemented; use min_rbf=0, max_rbf=1")
-    return _geometric_attn.apply(Q, K, V, coords, spreads, mask)
+    if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
+        raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
+    return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf)
 
 
 class GeoAttention(nn.Module):
@@ -91,11 +102,14 @@ class GeoAttention(nn.Module):
     pairwise C-alpha distance.  Constructor, parameters and forward follow
     old/old_scripts/encoder.py:43-121 (per-head QKV projections with bias,
     sigma = min_spread + exp(w), heads concatenated as a (d_k x heads)
-    interleave, bias-free output projection).  beta_weights is kept so that
-    state dicts line up, but does not enter the logits."""
+    interleave, bias-free output projection).  With legacy_logits=True the
+    logits are the reference module's (beta-weighted bias, [min_rbf, max_rbf]
+    pair mask); otherwise beta_weights is kept only so that state dicts line up."""
 
-    def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=0.0, max_rbf=1.00, learn_spreads=True):
+    def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=0.0, max_rbf=1.00, learn_spreads=True,
+                 legacy_logits=False):
         super().__init__()
+        self.legacy_logits = legacy_logits      # True: the reference module's beta-weighted bias and pair mask
         self.heads = heads
         self.d_model = d_model
         if self.d_model % self.heads != 0:
@@ -129,7 +143,10 @@ class GeoAttention(nn.Module):
         Q = torch.matmul(q.unsqueeze(1), self.q_proj.unsqueeze(0)) + self.q_bias.unsqueeze(0).unsqueeze(2)
         K = torch.matmul(k.unsqueeze(1), self.k_proj.unsqueeze(0)) + self.k_bias.unsqueeze(0).unsqueeze(2)
         V = torch.matmul(v.unsqueeze(1), self.v_proj.unsqueeze(0)) + self.v_bias.unsqueeze(0).unsqueeze(2)
-        out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, min_rbf=self.min_rbf, max_rbf=self.max_rbf)
+        if self.legacy_logits:
+            out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf, max_rbf=self.max_rbf)
+        else:
+            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask)
         out = out.to(q.dtype)
         out = out.permute(0, 2, 3, 1)                    # batch x N x d_k x heads
         out = out.reshape(batch, N, self.d_model)

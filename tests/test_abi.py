@@ -77,6 +77,10 @@ def test_attention_argument_validation():
     assert call(12, 55) == -6
     assert call(0, p + 2) == -5
     assert lib.proteus_geo_attn_fwd(p, p, p, p, p, None, p, p, 1, 2, 16, 48, 0, None) == -3
+    # legacy-logits entry point: same checks, plus beta and the rbf range
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, None, None, p, p, 1, 2, 16, 64, 0.0, 1.0, 0, None) == -1
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0.5, 0.5, 0, None) == -2
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 32, 0.0, 1.0, 0, None) == -3
 
 
 def test_check_raises_python_exceptions():
@@ -122,9 +126,9 @@ def test_operator_argument_errors_match_the_reference_surface():
     with pytest.raises(AssertionError):
         pa.geo_attn(Q, Q, Q, coords, torch.ones(3))
     with pytest.raises(NotImplementedError):
-        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), betas=torch.ones(2))
-    with pytest.raises(NotImplementedError):
-        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), None, min_rbf=0.1)
+        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), None, min_rbf=0.1)     # the pair mask needs betas
+    with pytest.raises(_lib.ProteusError):
+        pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), betas=torch.ones(2))    # legacy logits exist, but not on the CPU
 
 
 def test_wavefunction_embedding_module_schedule_and_parameters():

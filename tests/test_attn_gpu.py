@@ -210,3 +210,32 @@ def test_cfg5_sampled_rows(gpu):
     # size-independent property at full size: V = 1 -> O = 1
     O1, _ = run_gpu(gpu, Q, K, torch.ones_like(V), coords, sigma, None)
     assert np.abs(O1 - 1).max() < 1e-2
+
+
+def test_legacy_logits(gpu):
+    # the reference kernel's own logits S + beta*rbf_norm*|S| with its [min_rbf, max_rbf] pair mask
+    # (old/old_scripts/attn/geometric_attn.py:193-201), against the restated torch_attn oracle
+    Q, K, V, coords, sigma, mask = make(21, 2, 4, 333, maskfrac=0.15)
+    beta = torch.tensor([1.0, 0.5, 2.0, 0.1])
+    for min_rbf, max_rbf in ((0.0, 1.0), (0.001, 1.0)):
+        O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), return_lse=True,
+                           betas=beta.to(gpu), min_rbf=min_rbf, max_rbf=max_rbf)
+        torch.cuda.synchronize()
+        Or, Lr = c_oracle.geo_attn_legacy(Q.float().numpy(), K.float().numpy(), V.float().numpy(), coords.numpy(), sigma.numpy(),
+                                          beta.numpy(), mask.numpy(), min_rbf, max_rbf)
+        O, L = O.cpu().numpy().astype(np.float64), L.cpu().numpy().astype(np.float64)
+        # rows holding a pair whose rbf sits within 1e-4 (relative) of a threshold may legitimately flip: leave them out
+        d2 = ((coords[:, :, None].double() - coords[:, None].double()) ** 2).sum(-1)
+        rbf = torch.exp(-d2[:, None] / (2 * sigma.double()[None, :, None, None] ** 2))
+        edge = ((rbf - min_rbf).abs() < 1e-4 * max(min_rbf, 1e-30)).any(-1).numpy() if min_rbf > 0 else np.zeros(L.shape, bool)
+        fin = np.isfinite(Lr) & ~edge
+        assert (np.isneginf(L) == np.isneginf(Lr))[~edge].all()
+        assert np.abs(O - Or)[~edge].max() <= MAX_ABS_TOL
+        assert np.abs(L[fin] - Lr[fin]).max() <= LSE_TOL
+    # module: the reference's GeoAttention semantics (beta = exp(w), min_rbf default) are available on request
+    torch.manual_seed(1)
+    mod = pa.GeoAttention(d_model=128, heads=2, min_rbf=0.001, legacy_logits=True).to(gpu)
+    x = torch.randn(1, 70, 128)
+    with torch.no_grad():
+        y = mod(x.to(gpu), x.to(gpu), x.to(gpu), coords[:1, :70].to(gpu))
+    assert y.shape == (1, 70, 128) and torch.isfinite(y).all()

@@ -125,3 +125,28 @@ def test_row_subset_equals_full():
     assert np.array_equal(O[:, :, rows], Os) and np.array_equal(L[:, :, rows], Ls)
     Ot, Lt = torch_oracle.geo_attn_torch(Q, K, V, coords, sigma, mask, rows=rows.tolist(), dtype=torch.float64)
     assert np.abs(Ot.numpy() - Os).max() < 1e-11
+
+
+def test_legacy_logits_oracles():
+    # the reference kernel's own logits: C and torch statements agree, and beta = 0 with the full rbf range is
+    # plain scaled-dot-product attention with a key mask
+    Q, K, V, coords, sigma, mask = _case(8, maskfrac=0.25)
+    beta = torch.tensor([1.0, 0.3, 2.0])
+    Oc, Lc = c_oracle.geo_attn_legacy(Q.numpy(), K.numpy(), V.numpy(), coords.numpy(), sigma.numpy(), beta.numpy(), mask.numpy(), 0.001, 0.9)
+    Ot, Lt = torch_oracle.geo_attn_legacy_torch(Q, K, V, coords, sigma, beta, mask, 0.001, 0.9, dtype=torch.float64)
+    assert np.abs(Oc - Ot.numpy()).max() < 1e-11
+    fin = np.isfinite(Lc)
+    assert (np.isfinite(Lt.numpy()) == fin).all() and np.abs(Lc[fin] - Lt.numpy()[fin]).max() < 1e-11
+    O0, _ = c_oracle.geo_attn_legacy(Q.numpy(), K.numpy(), V.numpy(), coords.numpy(), sigma.numpy(), np.zeros(3, np.float32), mask.numpy(), 0.0, 1.0)
+    am = (~mask)[:, None, None, :].expand(-1, Q.shape[1], Q.shape[2], -1)
+    ref = F.scaled_dot_product_attention(Q.double(), K.double(), V.double(), attn_mask=am).numpy()
+    valid = ~mask.numpy()
+    for z in range(Q.shape[0]):
+        assert np.abs(O0[z][:, valid[z]] - ref[z][:, valid[z]]).max() < 1e-9
+    # identical coordinates: rbf = 1 -> rbf_norm = +1 -> logits S + beta |S|
+    same = torch.zeros_like(coords)
+    O1, _ = c_oracle.geo_attn_legacy(Q.numpy(), K.numpy(), V.numpy(), same.numpy(), sigma.numpy(), beta.numpy(), None, 0.0, 1.0)
+    S = torch.matmul(Q.double(), K.double().transpose(2, 3)) / 8
+    S = S + beta.double()[None, :, None, None] * S.abs()
+    ref1 = torch.matmul(torch.softmax(S, -1), V.double()).numpy()
+    assert np.abs(O1 - ref1).max() < 1e-10
