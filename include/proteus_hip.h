@@ -1,8 +1,8 @@
 /*
  * proteus_hip.h -- C ABI of libproteus_hip.so (gfx950 / MI355X).
  *
- * Two operators of jaimec00/proteusAI behind plain pointers and sizes:
- *   - the isotropic Wavefunction Embedding (WE) forward, and
+ * Operators of jaimec00/proteusAI behind plain pointers and sizes:
+ *   - the Wavefunction Embedding (WE) forward, isotropic and anisotropic, and
  *   - the RBF-scaled geometric flash-attention forward.
  *
  * Conventions shared by every entry point
@@ -95,6 +95,47 @@ int proteus_we_fwd_check(const float* coords, int coords_layout,
 
 int         proteus_we_num_variants(void);
 const char* proteus_we_variant_name(int tuning);
+
+/*
+ * Anisotropic (C-beta scaled, learnable wavenumber) Wavefunction Embedding
+ * forward: the variant WaveFunctionEmbedding(anisotropic=True) calls
+ *   utils/model_utils/wf_embedding/wf_embedding.py:41-42.
+ *
+ * Replaces the reference's native entry `wf_embedding_kernel.forward(coordsA,
+ * coordsB, cb_magnitudes, wavenumbers, out, d_cb, d_k)`
+ *   anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:57-61
+ * and its kernel
+ *   anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding_kernel.cu:30-224
+ * (paths under utils/model_utils/wf_embedding/).
+ *
+ * Semantics, for observer i, source j, index k, with R = a_i - a_j, r = |R|,
+ * A = (b_j . R)/r, u = r - cb_k A, phase = u k_k, over the pairs with both
+ * tokens unpadded and r != 0:
+ *     out [z,i,2k] = sum_j cos(phase)/r          out [z,i,2k+1] = sum_j sin(phase)/r
+ *     d_k [z,i,2k] = sum_j -sin(phase) u / r     d_k [z,i,2k+1] = sum_j  cos(phase) u / r
+ *     d_cb[z,i,2k] = sum_j  sin(phase) k_k A / r d_cb[z,i,2k+1] = sum_j -cos(phase) k_k A / r
+ *   A masked observer's rows are all zero.  Padding is an explicit byte mask,
+ *   as in proteus_we_fwd (the reference bakes x == 12345 into coordsA, :36).
+ *
+ *   coordsA, coordsB  [Z,3,N] or [Z,N,3] f32, both per coords_layout
+ *                     (positions; per-token C-beta direction vectors)
+ *   cb_magnitudes, wavenumbers  [K] f32
+ *   mask              [Z,N] u8, non-zero = padded; may be NULL
+ *   out, d_cb, d_k    [Z,N,2K] f32, 16-byte aligned
+ */
+int proteus_we_aniso_fwd(const float* coordsA, const float* coordsB, int coords_layout,
+                         const float* cb_magnitudes, const float* wavenumbers, const uint8_t* mask,
+                         float* out, float* d_cb, float* d_k,
+                         int Z, int N, int K, int tuning, void* stream);
+
+/* Validation half of proteus_we_aniso_fwd: same checks, no HIP call. */
+int proteus_we_aniso_fwd_check(const float* coordsA, const float* coordsB, int coords_layout,
+                               const float* cb_magnitudes, const float* wavenumbers, const uint8_t* mask,
+                               const float* out, const float* d_cb, const float* d_k,
+                               int Z, int N, int K, int tuning);
+
+int         proteus_we_aniso_num_variants(void);
+const char* proteus_we_aniso_variant_name(int tuning);
 
 /*
  * RBF-scaled geometric flash-attention forward.

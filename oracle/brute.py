@@ -38,6 +38,43 @@ def we_brute(coords, wavenumbers, mask=None):
     return out, cs, ss
 
 
+def we_aniso_brute(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None):
+    """coordsA, coordsB: Z x N x 3 nested lists; cb_magnitudes, wavenumbers: lists; mask: Z x N of bool.
+
+    Per pair: R = a_i - a_j, r = |R|, A = (b_j . R)/r, u = r - cb_k A, phase = u k_k
+    (tests/wf_embed/wf_embed_aniso_learnCB_learnK.py:127-149); out as in we_brute; the partials are
+    those of .../cb_scaling/learnable_wavenumbers/cuda/wf_embedding_kernel.cu:187-194.
+    Returns (out, d_cb, d_k), each Z x N x 2K.
+    """
+    Z, N, K = len(coordsA), len(coordsA[0]), len(wavenumbers)
+    out = [[[0.0] * (2 * K) for _ in range(N)] for _ in range(Z)]
+    d_cb = [[[0.0] * (2 * K) for _ in range(N)] for _ in range(Z)]
+    d_k = [[[0.0] * (2 * K) for _ in range(N)] for _ in range(Z)]
+    for z in range(Z):
+        for i in range(N):
+            if mask is not None and mask[z][i]:
+                continue
+            for j in range(N):
+                if mask is not None and mask[z][j]:
+                    continue
+                R = [coordsA[z][i][c] - coordsA[z][j][c] for c in range(3)]
+                r = math.sqrt(sum(x * x for x in R))
+                if r == 0.0:
+                    continue
+                A = sum(R[c] * coordsB[z][j][c] for c in range(3)) / r
+                for k in range(K):
+                    u = r - cb_magnitudes[k] * A
+                    ph = u * wavenumbers[k]
+                    real, imag = math.cos(ph) / r, math.sin(ph) / r
+                    out[z][i][2 * k] += real
+                    out[z][i][2 * k + 1] += imag
+                    d_k[z][i][2 * k] += -imag * u
+                    d_k[z][i][2 * k + 1] += real * u
+                    d_cb[z][i][2 * k] += imag * wavenumbers[k] * A
+                    d_cb[z][i][2 * k + 1] += -real * wavenumbers[k] * A
+    return out, d_cb, d_k
+
+
 def geo_attn_brute(Q, K, V, coords, sigma, key_padding_mask=None):
     """Q,K,V: Z x H x N x d nested lists. Returns (O, L) nested lists.
 

@@ -4,7 +4,7 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "_build", "liboracle.so")
-SOURCES = ["we_oracle.c", "geo_attn_oracle.c"]
+SOURCES = ["we_oracle.c", "we_aniso_oracle.c", "geo_attn_oracle.c"]
 
 
 def build(force: bool = True) -> str:

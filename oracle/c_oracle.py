@@ -17,7 +17,8 @@ def lib():
     global _lib
     if _lib is None:
         path = _build.LIB
-        if not os.path.exists(path):
+        srcs = [os.path.join(_build.HERE, f) for f in _build.SOURCES]
+        if not os.path.exists(path) or any(os.path.getmtime(f) > os.path.getmtime(path) for f in srcs):
             _build.build()
         _lib = ctypes.CDLL(path)
     return _lib
@@ -61,6 +62,34 @@ def we(coords, wavenumbers, mask=None, rows=None, precision="f64"):
        ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K), _p(r, ctypes.c_int), ctypes.c_int(R),
        _p(out, ct), _p(cs, ct), _p(ss, ct))
     return out, cs, ss
+
+
+def we_aniso(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, rows=None):
+    """coordsA, coordsB [Z,N,3], cb_magnitudes, wavenumbers [K], mask [Z,N] bool (True = padded).
+
+    Returns (out, d_cb, d_k), each [Z,R,2K] float64, for the selected rows.
+    """
+    a = np.ascontiguousarray(np.asarray(coordsA, dtype=np.float32))
+    b = np.ascontiguousarray(np.asarray(coordsB, dtype=np.float32))
+    w = np.ascontiguousarray(np.asarray(wavenumbers, dtype=np.float32))
+    cb = np.ascontiguousarray(np.asarray(cb_magnitudes, dtype=np.float32))
+    Z, N, three = a.shape
+    assert three == 3 and b.shape == a.shape and cb.shape == w.shape and w.ndim == 1
+    K = int(w.shape[0])
+    m = None if mask is None else np.ascontiguousarray(np.asarray(mask).astype(np.uint8))
+    if m is not None:
+        assert m.shape == (Z, N)
+    r, R = _rows(rows, N)
+    out = np.empty((Z, R, 2 * K), np.float64)
+    d_cb = np.empty_like(out)
+    d_k = np.empty_like(out)
+    fn = lib().we_aniso_oracle_f64
+    fn.restype = None
+    cf, cd = ctypes.c_float, ctypes.c_double
+    fn(_p(a, cf), _p(b, cf), _p(cb, cf), _p(w, cf), _p(m, ctypes.c_uint8),
+       ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K), _p(r, ctypes.c_int), ctypes.c_int(R),
+       _p(out, cd), _p(d_cb, cd), _p(d_k, cd))
+    return out, d_cb, d_k
 
 
 def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, rows=None):

@@ -56,6 +56,43 @@ def we_torch(coords, wavenumbers, mask=None, rows=None, row_chunk=None, dtype=to
     return out, cs, ss
 
 
+def we_aniso_torch(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, dtype=torch.float64):
+    """Anisotropic (C-beta scaled) wavefunction embedding, dense and differentiable in cb_magnitudes
+    and wavenumbers.
+
+    Follows tests/wf_embed/wf_embed_aniso_learnCB_learnK.py:117-163 (wf_embedding_torch):
+    R = a_i - a_j; R_unit = R/|R| (0 where |R| = 0); distsB = R_unit . (b_j cb_k);
+    phases = (|R| - distsB) k; masked = m_i | m_j | |R| == 0; magnitudes = 1/where(masked, inf, |R|);
+    features = stack([sum_j mag cos, sum_j mag sin], -1).view(Z, N, 2K).
+    """
+    a = coordsA.to(dtype)
+    b = coordsB.to(dtype)
+    cb = cb_magnitudes.to(dtype)
+    wn = wavenumbers.to(dtype)
+    Z, N, _ = a.shape
+    K = wn.shape[0]
+    mask = torch.zeros(Z, N, dtype=torch.bool) if mask is None else mask.bool()
+    R = a[:, :, None, :] - a[:, None, :, :]                                   # Z x N x N x 3
+    R_norm = torch.linalg.vector_norm(R, dim=3, keepdim=True)                 # Z x N x N x 1
+    R_unit = R / torch.where(R_norm == 0, torch.full_like(R_norm, float("inf")), R_norm)
+    b_scaled = b[:, :, None, :] * cb[None, None, :, None]                     # Z x N x K x 3
+    distsB = torch.sum(R_unit[:, :, :, None, :] * b_scaled[:, None, :, :, :], dim=4)   # Z x N x N x K
+    phases = (R_norm - distsB) * wn[None, None, None, :]
+    m = mask[:, :, None, None] | mask[:, None, :, None] | (R_norm == 0)
+    mag = 1 / torch.where(m, torch.full_like(R_norm, float("inf")), R_norm)
+    real = (mag * torch.cos(phases)).sum(dim=2)
+    imag = (mag * torch.sin(phases)).sum(dim=2)
+    return torch.stack([real, imag], dim=-1).view(Z, N, 2 * K)
+
+
+def we_aniso_backward_torch(dO, d_cb, d_k):
+    """anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:65-79: contract the per-token
+    partial derivatives with dO over batch and tokens, then add the real and imaginary halves."""
+    g_cb = (dO * d_cb).sum(dim=(0, 1))
+    g_k = (dO * d_k).sum(dim=(0, 1))
+    return g_cb[0::2] + g_cb[1::2], g_k[0::2] + g_k[1::2]
+
+
 def we_backward_torch(dO, cos_sums, sin_sums):
     """d(loss)/d(wavenumbers): isotropic/cuda/wf_embedding.py:64-83."""
     real_dO = dO[:, :, 0::2]

@@ -16,6 +16,7 @@ COORDS_AOS = 1
 SYMBOLS = [
     "proteus_version", "proteus_strerror",
     "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_num_variants", "proteus_we_variant_name",
+    "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_probe_valu_rate", "proteus_probe_sincos",
@@ -49,6 +50,13 @@ def load():
     lib.proteus_we_num_variants.restype = ci
     lib.proteus_we_variant_name.restype = ctypes.c_char_p
     lib.proteus_we_variant_name.argtypes = [ci]
+    lib.proteus_we_aniso_fwd.restype = ci
+    lib.proteus_we_aniso_fwd.argtypes = [vp, vp, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.proteus_we_aniso_fwd_check.restype = ci
+    lib.proteus_we_aniso_fwd_check.argtypes = [vp, vp, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci]
+    lib.proteus_we_aniso_num_variants.restype = ci
+    lib.proteus_we_aniso_variant_name.restype = ctypes.c_char_p
+    lib.proteus_we_aniso_variant_name.argtypes = [ci]
     lib.proteus_geo_attn_fwd.restype = ci
     lib.proteus_geo_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     lib.proteus_geo_attn_legacy_fwd.restype = ci
@@ -81,6 +89,11 @@ def check(rc: int, what: str):
 def we_variants():
     lib = load()
     return [lib.proteus_we_variant_name(i).decode() for i in range(lib.proteus_we_num_variants())]
+
+
+def we_aniso_variants():
+    lib = load()
+    return [lib.proteus_we_aniso_variant_name(i).decode() for i in range(lib.proteus_we_aniso_num_variants())]
 
 
 def geo_attn_variants():

@@ -1,14 +1,16 @@
-"""Wavefunction Embedding operator and module on the HIP kernel.
+"""Wavefunction Embedding operators and module on the HIP kernels.
 
-Mirrors the reference's Python surface for the isotropic path:
-  wf_embedding(...) / _wf_embedding      utils/model_utils/wf_embedding/isotropic/cuda/wf_embedding.py:18-83
-  WaveFunctionEmbedding                  utils/model_utils/wf_embedding/wf_embedding.py:24-46
-plus `we_forward`, which also returns the per-token cos/sin sums.
+Mirrors the reference's Python surface (paths under utils/model_utils/wf_embedding/):
+  wf_embedding(...) / _wf_embedding      isotropic/cuda/wf_embedding.py:18-83
+  wf_embedding_learnCB(...)              anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:16-79
+  WaveFunctionEmbedding                  wf_embedding.py:24-49
+plus `we_forward` / `we_aniso_forward`, which also return what the kernels save for the backward.
 """
 import torch
 import torch.nn as nn
 
 from . import _lib
+from .cb_utils import get_coords
 
 
 def we_forward(coords, wavenumbers, mask=None, tuning: int = 0):
@@ -85,12 +87,85 @@ def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None
     return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask)
 
 
+def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tuning: int = 0):
+    """out, d_cb, d_k = we_aniso_forward(coordsA [Z,N,3], coordsB [Z,N,3], cb_magnitudes [K], wavenumbers [K], mask).
+
+    coordsA: token positions; coordsB: per-token C-beta direction vectors (relative to the token);
+    mask [Z,N] bool, True = padded (None = nothing padded).  All outputs float32 [Z,N,2K], cos/real
+    terms at even and sin/imag terms at odd indices: the embedding and its per-token partial
+    derivatives with respect to cb_magnitudes and wavenumbers
+    (anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding_kernel.cu:163-206).
+    """
+    if coordsA.dim() != 3 or coordsA.size(2) != 3:
+        raise ValueError(f"coordsA must be of shape (batch, N, 3), not {tuple(coordsA.shape)}")
+    if tuple(coordsB.shape) != tuple(coordsA.shape):
+        raise ValueError(f"coordsB must have coordsA's shape {tuple(coordsA.shape)}, not {tuple(coordsB.shape)}")
+    if wavenumbers.dim() != 1 or tuple(cb_magnitudes.shape) != tuple(wavenumbers.shape):
+        raise ValueError(f"cb_magnitudes and wavenumbers must both be of shape (K,), not "
+                         f"{tuple(cb_magnitudes.shape)} and {tuple(wavenumbers.shape)}")
+    if not coordsA.is_cuda:
+        raise _lib.ProteusError("we_aniso_forward needs tensors on the GPU (there is no CPU path)")
+    lib = _lib.load()
+    dev = coordsA.device
+    a = coordsA.detach().to(torch.float32).contiguous()
+    b = coordsB.detach().to(device=dev, dtype=torch.float32).contiguous()
+    w = wavenumbers.detach().to(device=dev, dtype=torch.float32).contiguous()
+    cb = cb_magnitudes.detach().to(device=dev, dtype=torch.float32).contiguous()
+    Z, N, _ = a.shape
+    K = w.shape[0]
+    m = None
+    if mask is not None:
+        if tuple(mask.shape) != (Z, N):
+            raise ValueError(f"mask must be of shape ({Z}, {N}), not {tuple(mask.shape)}")
+        m = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
+    out = torch.empty(Z, N, 2 * K, dtype=torch.float32, device=dev)
+    d_cb = torch.empty_like(out)
+    d_k = torch.empty_like(out)
+    if Z == 0 or N == 0 or K == 0:
+        return out, d_cb, d_k
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.proteus_we_aniso_fwd(a.data_ptr(), b.data_ptr(), _lib.COORDS_AOS, cb.data_ptr(), w.data_ptr(),
+                                      None if m is None else m.data_ptr(),
+                                      out.data_ptr(), d_cb.data_ptr(), d_k.data_ptr(),
+                                      Z, N, K, int(tuning), stream)
+    _lib.check(rc, "proteus_we_aniso_fwd")
+    return out, d_cb, d_k
+
+
+class _wf_embedding_learnCB(torch.autograd.Function):
+    """Forward on the HIP kernel; the backward contracts the saved per-token partial derivatives with dO
+    (anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:65-79).  No gradient flows to the
+    coordinates, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask):
+        out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask)
+        ctx.save_for_backward(d_cb.to(cb_magnitudes.dtype), d_k.to(wavenumbers.dtype))
+        return out.to(coordsA.dtype)
+
+    @staticmethod
+    def backward(ctx, dO):
+        d_cb, d_k = ctx.saved_tensors
+        g_cb = (dO * d_cb).sum(dim=(0, 1))
+        g_cb = g_cb[0::2] + g_cb[1::2]
+        g_k = (dO * d_k).sum(dim=(0, 1))
+        g_k = g_k[0::2] + g_k[1::2]
+        return None, None, g_cb, g_k, None
+
+
+def wf_embedding_learnCB(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None):
+    """Same call as the reference's anisotropic wf_embedding
+    (anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:16)."""
+    return _wf_embedding_learnCB.apply(coordsA, coordsB, cb_magnitudes, wavenumbers, mask)
+
+
 class WaveFunctionEmbedding(nn.Module):
-    """Same constructor and forward as utils/model_utils/wf_embedding/wf_embedding.py:24-46.
+    """Same constructor and forward as utils/model_utils/wf_embedding/wf_embedding.py:24-49.
 
     The wavelength schedule follows the code (torch.logspace, endpoint
-    inclusive), the parameter holds log(wavenumber).  Only the isotropic branch
-    exists here; anisotropic=True (the reference default) raises.
+    inclusive), the parameter holds log(wavenumber).  anisotropic=True (the
+    reference default) takes the C-beta scaled kernel and needs coords_beta.
     """
 
     def __init__(self, d_wf=512, min_wl=4.0, max_wl=35.0, base_wl=20.0, anisotropic=True, learn_wl=False, learn_aa=False):
@@ -106,6 +181,11 @@ class WaveFunctionEmbedding(nn.Module):
 
     def forward(self, coords_alpha, coords_beta=None, key_padding_mask=None):
         if self.aniso:
-            raise NotImplementedError("the anisotropic (C-beta scaled) embedding is not implemented; "
-                                      "construct with anisotropic=False")
+            if coords_beta is None:
+                raise ValueError("the anisotropic embedding needs coords_beta (see get_CaCb_coords)")
+            return wf_embedding_learnCB(coords_alpha, coords_beta, self.aa_magnitudes, self.get_wavenumbers(),
+                                        mask=key_padding_mask)
         return wf_embedding(coords_alpha, self.get_wavenumbers(), magnitude_type=1, dropout_p=0.0, mask=key_padding_mask)
+
+    def get_CaCb_coords(self, coords, chain_idxs=None, norm=False):
+        return get_coords(coords, chain_idxs, norm)

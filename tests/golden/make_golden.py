@@ -43,6 +43,29 @@ def we_golden():
              out=np.array(out), cos_sums=np.array(cs), sin_sums=np.array(ss))
 
 
+def we_aniso_golden():
+    rng = np.random.default_rng(20240609)
+    Z, N, K = 2, 21, 5
+    steps = rng.normal(size=(Z, N, 3))
+    steps = 3.8 * steps / np.linalg.norm(steps, axis=-1, keepdims=True)
+    a = np.cumsum(steps, axis=1).astype(np.float32)
+    a[0, 9] = a[0, 2]                        # a coincident pair
+    b = rng.normal(size=(Z, N, 3))
+    b = (b / np.linalg.norm(b, axis=-1, keepdims=True)).astype(np.float32)
+    b[1, 0] = 0                              # chain ends carry no C-beta vector
+    wl = 3.7 + (20 - 3.7) * (20 ** (np.arange(K) / K) - 1) / 19
+    wn = (2 * np.pi / wl).astype(np.float32)
+    cb = rng.uniform(0.5, 2.5, K).astype(np.float32)
+    cb[3] = -cb[3]
+    mask = np.zeros((Z, N), bool)
+    mask[1, 16:] = True
+    mask[1, 5] = True
+    out, d_cb, d_k = brute.we_aniso_brute(a.astype(np.float64).tolist(), b.astype(np.float64).tolist(),
+                                          cb.astype(np.float64).tolist(), wn.astype(np.float64).tolist(), mask.tolist())
+    np.savez(os.path.join(HERE, "we_aniso_small.npz"), coordsA=a, coordsB=b, cb_magnitudes=cb, wavenumbers=wn,
+             mask=mask, out=np.array(out), d_cb=np.array(d_cb), d_k=np.array(d_k))
+
+
 def attn_golden():
     rng = np.random.default_rng(20240608)
     Z, H, N, d = 2, 2, 20, 64
@@ -65,5 +88,6 @@ def attn_golden():
 
 if __name__ == "__main__":
     we_golden()
+    we_aniso_golden()
     attn_golden()
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))

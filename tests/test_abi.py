@@ -57,6 +57,28 @@ def test_we_argument_validation_happens_before_any_hip_call():
     assert lib.proteus_we_fwd(p, 7, p, None, p, p, p, 1, 8, 4, 0, None) == -4
 
 
+def test_we_aniso_argument_validation():
+    lib = _lib.load()
+    p = 0x1000
+    ok = dict(a=p, b=p, layout=1, cb=p, wn=p, mask=None, out=p, dcb=p, dk=p, Z=1, N=8, K=4, tuning=0)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return lib.proteus_we_aniso_fwd_check(a["a"], a["b"], a["layout"], a["cb"], a["wn"], a["mask"],
+                                              a["out"], a["dcb"], a["dk"], a["Z"], a["N"], a["K"], a["tuning"])
+    assert call() == 0
+    for name in ("a", "b", "cb", "wn", "out", "dcb", "dk"):
+        assert call(**{name: None}) == -1
+    for name in ("Z", "N", "K"):
+        assert call(**{name: 0}) == -2
+    assert call(N=(1 << 22) + 1) == -2 and call(K=4097) == -2
+    assert call(layout=5) == -4
+    assert call(dk=p + 8) == -5
+    assert call(tuning=len(_lib.we_aniso_variants())) == -6
+    assert lib.proteus_we_aniso_fwd(p, None, 1, p, p, None, p, p, p, 1, 8, 4, 0, None) == -1
+    assert _lib.we_aniso_variants()[0] == "auto"
+
+
 def test_attention_argument_validation():
     lib = _lib.load()
     p = 0x1000
@@ -140,8 +162,15 @@ def test_wavefunction_embedding_module_schedule_and_parameters():
     assert torch.all(wl[1:] > wl[:-1])
     assert m.wavenumbers.requires_grad and not m.aa_magnitudes.requires_grad
     assert set(dict(m.named_parameters())) == {"wavenumbers", "aa_magnitudes"}
-    with pytest.raises(NotImplementedError):
+    # the default module is the anisotropic one: it needs coords_beta and, like every operator, the GPU
+    with pytest.raises(ValueError):
+        pa.WaveFunctionEmbedding()(torch.randn(1, 4, 3))
+    with pytest.raises(_lib.ProteusError):
         pa.WaveFunctionEmbedding()(torch.randn(1, 4, 3), torch.randn(1, 4, 3))
+    with pytest.raises(ValueError):
+        pa.wf_embedding_learnCB(torch.randn(1, 4, 3), torch.randn(1, 5, 3), torch.ones(3), torch.ones(3))
+    with pytest.raises(ValueError):
+        pa.wf_embedding_learnCB(torch.randn(1, 4, 3), torch.randn(1, 4, 3), torch.ones(2), torch.ones(3))
 
 
 def test_geo_attention_module_parameters():

@@ -1,0 +1,180 @@
+"""GPU parity tests of the anisotropic (C-beta scaled) Wavefunction Embedding forward: the HIP kernel,
+called through the C ABI, against the fp64 CPU oracle on the same seeded inputs.
+
+Bar: relative L2 error <= 1e-4 for out, d_cb and d_k (each tensor separately), the fp32 bar of the
+isotropic embedding."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import proteusai_amd as pa
+from oracle import c_oracle, torch_oracle
+from proteusai_amd import _lib, synth
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-4
+NAMES = ("out", "d_cb", "d_k")
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    nb = np.linalg.norm(b)
+    return float(np.linalg.norm(a - b) / nb) if nb > 0 else float(np.linalg.norm(a - b))
+
+
+def inputs(N, seed, batch=1, K=256, pad=0.0, compact=False):
+    coords, _ = synth.we_inputs(N, seed=seed, batch=batch, compact=compact)
+    g = torch.Generator().manual_seed(1000 + seed)
+    b = torch.randn(batch, N, 3, generator=g)
+    b = b / b.norm(dim=-1, keepdim=True)
+    wn = synth.wavenumbers(2 * K)
+    cb = 0.5 + 2.0 * torch.rand(K, generator=g)
+    mask = None
+    if pad > 0:
+        mask = torch.rand(batch, N, generator=g) < pad
+    return coords, b, cb, wn, mask
+
+
+def run_gpu(gpu, a, b, cb, wn, mask=None, tuning=0):
+    res = pa.we_aniso_forward(a.to(gpu), b.to(gpu), cb.to(gpu), wn.to(gpu), None if mask is None else mask.to(gpu),
+                              tuning=tuning)
+    torch.cuda.synchronize()
+    return tuple(t.cpu().numpy() for t in res)
+
+
+def check(got, a, b, cb, wn, mask=None, rows=None, what=""):
+    m = None if mask is None else mask.numpy()
+    ref = c_oracle.we_aniso(a.numpy(), b.numpy(), cb.numpy(), wn.numpy(), m, rows=rows)
+    sel = slice(None) if rows is None else np.asarray(rows)
+    for g, r, name in zip(got, ref, NAMES):
+        g = g[:, sel]
+        assert np.isfinite(g).all(), f"{what} {name}: non-finite values"
+        e = rel_l2(g, r)
+        assert e <= REL_L2_TOL, f"{what} {name}: rel-L2 {e:.3e}"
+
+
+def test_cfg1_full(gpu):
+    a, b, cb, wn, _ = inputs(512, seed=1)
+    check(run_gpu(gpu, a, b, cb, wn), a, b, cb, wn, what="cfg1")
+
+
+def test_golden_fixture(gpu, golden_dir):
+    g = np.load(os.path.join(golden_dir, "we_aniso_small.npz"))
+    got = run_gpu(gpu, *(torch.from_numpy(g[k]) for k in ("coordsA", "coordsB", "cb_magnitudes", "wavenumbers", "mask")))
+    for x, key in zip(got, NAMES):
+        assert rel_l2(x, g[key]) <= REL_L2_TOL, key
+        assert (x[g["mask"]] == 0).all(), key
+
+
+@pytest.mark.parametrize("tuning", range(1, 5))
+def test_every_variant(gpu, tuning):
+    assert len(_lib.we_aniso_variants()) == 5
+    a, b, cb, wn, mask = inputs(333, seed=3, batch=2, K=40, pad=0.2)
+    check(run_gpu(gpu, a, b, cb, wn, mask, tuning=tuning), a, b, cb, wn, mask, what=_lib.we_aniso_variants()[tuning])
+
+
+@pytest.mark.parametrize("N", [1, 2, 63, 64, 65, 257, 700])
+def test_ragged_lengths(gpu, N):
+    a, b, cb, wn, _ = inputs(N, seed=10 + N, batch=2, K=32)
+    got = run_gpu(gpu, a, b, cb, wn)
+    if N == 1:
+        assert all((x == 0).all() for x in got)
+    else:
+        check(got, a, b, cb, wn, what=f"N={N}")
+
+
+@pytest.mark.parametrize("K", [1, 3, 16, 35, 65])
+def test_odd_wavenumber_counts(gpu, K):
+    a, b, cb, wn, mask = inputs(200, seed=20 + K, K=K, pad=0.1)
+    check(run_gpu(gpu, a, b, cb, wn, mask), a, b, cb, wn, mask, what=f"K={K}")
+
+
+def test_masks_padded_content_and_coincident_points(gpu):
+    a, b, cb, wn, mask = inputs(300, seed=5, batch=2, K=24, pad=0.3)
+    mask[0, 10] = False
+    mask[0, 11] = False
+    a[0, 11] = a[0, 10]                                   # a coincident pair is dropped like the self pair
+    got = run_gpu(gpu, a, b, cb, wn, mask)
+    check(got, a, b, cb, wn, mask, what="masked")
+    for x in got:
+        assert (x[mask.numpy()] == 0).all()
+    a2, b2 = a.clone(), b.clone()
+    a2[mask] = float("nan")
+    b2[mask] = float("nan")
+    got2 = run_gpu(gpu, a2, b2, cb, wn, mask)
+    for x, y in zip(got, got2):
+        np.testing.assert_array_equal(x, y)               # what padded tokens hold cannot matter
+    all_pad = torch.ones(2, 300, dtype=torch.bool)
+    assert all((x == 0).all() for x in run_gpu(gpu, a, b, cb, wn, all_pad))
+
+
+def test_zero_cb_equals_isotropic_kernel(gpu):
+    a, b, cb, wn, mask = inputs(400, seed=6, K=64, pad=0.1)
+    out, d_cb, d_k = run_gpu(gpu, a, b, torch.zeros_like(cb), wn, mask)
+    iso, cs, ss = (t.cpu().numpy() for t in pa.we_forward(a.to(gpu), wn.to(gpu), mask.to(gpu)))
+    assert rel_l2(out, iso) <= 1e-5
+    assert rel_l2(d_k[..., 1::2], cs) <= 1e-5 and rel_l2(d_k[..., 0::2], -ss) <= 1e-5
+
+
+def test_large_phases_and_far_offsets(gpu):
+    # phases of hundreds of revolutions, far from the origin: the explicit range reduction must hold up.
+    # (The scale is bounded by fp32 itself: a phase of P radians carries an error of about P * 2^-24 from
+    # the rounding of r alone, in any fp32 implementation.)
+    a, b, cb, wn, _ = inputs(256, seed=7, K=16)
+    a = a * 10 + torch.tensor([3000.0, -2000.0, 500.0])
+    check(run_gpu(gpu, a, b, cb * 3, wn), a, b, cb * 3, wn, what="far")
+
+
+def test_cfg2_sampled_rows(gpu):
+    # N=16384, K=256: 48 sampled observers against the oracle, plus the cb = 0 identity on every row
+    a, b, cb, wn, _ = inputs(16384, seed=2, compact=True)
+    got = run_gpu(gpu, a, b, cb, wn)
+    rows = np.random.default_rng(0).choice(16384, 48, replace=False)
+    check(got, a, b, cb, wn, rows=np.sort(rows), what="cfg2")
+
+
+def test_autograd_function_and_module(gpu):
+    a, b, cb, wn, mask = inputs(96, seed=8, batch=2, K=12, pad=0.2)
+    tcb = cb.to(gpu).requires_grad_(True)
+    twn = wn.to(gpu).requires_grad_(True)
+    out = pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), tcb, twn, mask.to(gpu))
+    dO = torch.randn(out.shape, generator=torch.Generator().manual_seed(3)).to(gpu)
+    out.backward(dO)
+    rcb = cb.double().requires_grad_(True)
+    rwn = wn.double().requires_grad_(True)
+    ref = torch_oracle.we_aniso_torch(a, b, rcb, rwn, mask)
+    ref.backward(dO.cpu().double())
+    assert rel_l2(out.detach().cpu().numpy(), ref.detach().numpy()) <= REL_L2_TOL
+    assert rel_l2(tcb.grad.cpu().numpy(), rcb.grad.numpy()) <= REL_L2_TOL
+    assert rel_l2(twn.grad.cpu().numpy(), rwn.grad.numpy()) <= REL_L2_TOL
+
+    mod = pa.WaveFunctionEmbedding(d_wf=24, learn_wl=True, learn_aa=True).to(gpu)
+    bb = torch.randn(2, 96, 3, 3, generator=torch.Generator().manual_seed(4)).to(gpu)
+    ca, cbv = mod.get_CaCb_coords(bb, norm=True)
+    y = mod(ca, cbv, mask.to(gpu))
+    y.square().sum().backward()
+    assert y.shape == (2, 96, 24) and mod.aa_magnitudes.grad is not None and mod.wavenumbers.grad is not None
+    r = torch_oracle.we_aniso_torch(ca.cpu(), cbv.cpu(), mod.aa_magnitudes.detach().cpu(), mod.get_wavenumbers().detach().cpu(), mask)
+    assert rel_l2(y.detach().cpu().numpy(), r.numpy()) <= REL_L2_TOL
+
+
+def test_raw_c_abi_soa_layout_and_stream(gpu):
+    a, b, cb, wn, mask = inputs(150, seed=9, batch=2, K=20, pad=0.15)
+    lib = _lib.load()
+    ta = a.transpose(1, 2).contiguous().to(gpu)           # [Z,3,N], what the reference wrapper hands its kernel
+    tb = b.transpose(1, 2).contiguous().to(gpu)
+    m = mask.to(gpu).view(torch.uint8)
+    tcb, twn = cb.to(gpu), wn.to(gpu)
+    outs = [torch.full((2, 150, 40), float("nan"), device=gpu) for _ in range(3)]
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    rc = lib.proteus_we_aniso_fwd(ta.data_ptr(), tb.data_ptr(), _lib.COORDS_SOA, tcb.data_ptr(), twn.data_ptr(),
+                                  m.data_ptr(), outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(),
+                                  2, 150, 20, 0, st.cuda_stream)
+    assert rc == 0
+    st.synchronize()
+    check(tuple(o.cpu().numpy() for o in outs), a, b, cb, wn, mask, what="soa")
