@@ -97,6 +97,21 @@ int         proteus_we_num_variants(void);
 const char* proteus_we_variant_name(int tuning);
 
 /*
+ * proteus_we_fwd with the source weight m(r) of the reference's other
+ * `magnitude_type` values (isotropic/cuda/wf_embedding_kernel.cu:192-206):
+ *   0: m = 1    1: m = 1/r (the same as proteus_we_fwd)    2: m = 1/log2(r)    3: m = 1/sqrt(r)
+ *     out[z,i,2k], out[z,i,2k+1] = sum_j valid * m cos(k_k r), sum_j valid * m sin(k_k r)
+ *     cos_sums, sin_sums         = sum_j valid * m r cos(k_k r), ... sin   (kernel.cu:237-238)
+ * Any other magnitude_type returns PROTEUS_ERR_UNSUPPORTED.  The reference's
+ * in-kernel dropout (dropout_p != 0, kernel.cu:227-232) draws a fresh seed per call
+ * (isotropic/cuda/wf_embedding.py:48-49) and is not provided.
+ */
+int proteus_we_legacy_fwd(const float* coords, int coords_layout,
+                          const float* wavenumbers, const uint8_t* mask,
+                          float* out, float* cos_sums, float* sin_sums,
+                          int Z, int N, int K, int magnitude_type, void* stream);
+
+/*
  * Anisotropic (C-beta scaled, learnable wavenumber) Wavefunction Embedding
  * forward: the variant WaveFunctionEmbedding(anisotropic=True) calls
  *   utils/model_utils/wf_embedding/wf_embedding.py:41-42.

@@ -36,8 +36,10 @@ def _rows(rows, N):
     return r, int(r.shape[0])
 
 
-def we(coords, wavenumbers, mask=None, rows=None, precision="f64"):
+def we(coords, wavenumbers, mask=None, rows=None, precision="f64", mag_type=1):
     """coords [Z,N,3], wavenumbers [K], mask [Z,N] bool (True = padded).
+
+    mag_type other than 1 (the reference's other source weights) is evaluated in f64 only.
 
     Returns (out [Z,R,2K], cos_sums [Z,R,K], sin_sums [Z,R,K]) for the selected
     rows (all rows when rows is None), float64 for precision 'f64' and float32
@@ -57,6 +59,14 @@ def we(coords, wavenumbers, mask=None, rows=None, precision="f64"):
     out = np.empty((Z, R, 2 * K), dt)
     cs = np.empty((Z, R, K), dt)
     ss = np.empty((Z, R, K), dt)
+    if mag_type != 1:
+        assert precision == "f64" and mag_type in (0, 2, 3)
+        fn = lib().we_oracle_mag_f64
+        fn.restype = None
+        fn(_p(c, ctypes.c_float), _p(w, ctypes.c_float), _p(m, ctypes.c_uint8),
+           ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K), ctypes.c_int(mag_type),
+           _p(r, ctypes.c_int), ctypes.c_int(R), _p(out, ct), _p(cs, ct), _p(ss, ct))
+        return out, cs, ss
     fn.restype = None
     fn(_p(c, ctypes.c_float), _p(w, ctypes.c_float), _p(m, ctypes.c_uint8),
        ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K), _p(r, ctypes.c_int), ctypes.c_int(R),

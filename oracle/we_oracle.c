@@ -101,3 +101,44 @@ void we_oracle_f32(const float* coords, const float* wn, const uint8_t* mask, in
         free(acc);
     }
 }
+
+/*
+ * The reference's other source weights (isotropic/cuda/wf_embedding_kernel.cu:192-206;
+ * dense statement tests/wf_embed/wf_embed.py:108-116):
+ *   mag_type 0: m = 1   1: m = 1/d   2: m = 1/log2(d)   3: m = 1/sqrt(d)
+ *   out = sum_j m cos, m sin ;  cos_sums, sin_sums = sum_j (m d) cos, (m d) sin   kernel.cu:237-238
+ */
+void we_oracle_mag_f64(const float* coords, const float* wn, const uint8_t* mask, int Z, int N, int K,
+                       int mag_type, const int* rows, int nrows,
+                       double* out, double* cs, double* ss)
+{
+    #pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int z = 0; z < Z; ++z)
+    for (int rr = 0; rr < nrows; ++rr) {
+        const int i = rows ? rows[rr] : rr;
+        const float* c = coords + (size_t)z * N * 3;
+        const uint8_t* m = mask ? mask + (size_t)z * N : NULL;
+        double* o = out + ((size_t)z * nrows + rr) * 2 * K;
+        double* pc = cs + ((size_t)z * nrows + rr) * K;
+        double* ps = ss + ((size_t)z * nrows + rr) * K;
+        for (int k = 0; k < K; ++k) { o[2*k] = o[2*k+1] = pc[k] = ps[k] = 0.0; }
+        if (m && m[i]) continue;
+        const double xi = c[3*i], yi = c[3*i+1], zi = c[3*i+2];
+        for (int j = 0; j < N; ++j) {
+            if (m && m[j]) continue;
+            const double dx = xi - c[3*j], dy = yi - c[3*j+1], dz = zi - c[3*j+2];
+            const double d2 = dx*dx + dy*dy + dz*dz;
+            if (d2 == 0.0) continue;
+            const double d = sqrt(d2);
+            double w = 1.0;
+            if (mag_type == 1) w = 1.0 / d;
+            if (mag_type == 2) w = 1.0 / log2(d);
+            if (mag_type == 3) w = 1.0 / sqrt(d);
+            for (int k = 0; k < K; ++k) {
+                const double ph = d * (double)wn[k];
+                const double co = cos(ph), si = sin(ph);
+                o[2*k] += co * w; o[2*k+1] += si * w; pc[k] += co * w * d; ps[k] += si * w * d;
+            }
+        }
+    }
+}

@@ -15,7 +15,7 @@ COORDS_AOS = 1
 # every symbol include/proteus_hip.h declares
 SYMBOLS = [
     "proteus_version", "proteus_strerror",
-    "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_num_variants", "proteus_we_variant_name",
+    "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_num_variants", "proteus_we_variant_name",
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
@@ -45,6 +45,8 @@ def load():
     lib.proteus_strerror.argtypes = [ci]
     lib.proteus_we_fwd.restype = ci
     lib.proteus_we_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.proteus_we_legacy_fwd.restype = ci
+    lib.proteus_we_legacy_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
     lib.proteus_we_fwd_check.restype = ci
     lib.proteus_we_fwd_check.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci]
     lib.proteus_we_num_variants.restype = ci

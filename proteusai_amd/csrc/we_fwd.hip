@@ -44,7 +44,10 @@ __device__ __forceinline__ float sgpr(float v) {
 // Inner loop: every lane (observer) against the nk staged sources, KT wavenumbers each.
 // FRACT: reduce the phase to [0,1) revolutions before v_sin/v_cos (needed only when it can exceed
 // the +-256 revolutions those instructions accept).
-template <int KT, bool FRACT>
+// MAG: the weight m(r) of a source (isotropic/cuda/wf_embedding_kernel.cu:192-206): 0: 1, 1: 1/r,
+// 2: 1/log2(r), 3: 1/sqrt(r).  The embedding sums m cos, m sin and the saved sums m r cos, m r sin
+// (kernel.cu:224-238); for MAG 1 the latter weight is 1 and the accumulation a plain add.
+template <int KT, bool FRACT, int MAG>
 __device__ __forceinline__ void stream_sources(const float4* s_keys, const int first, const int step, const int nk,
                                                const float xi, const float yi, const float zi,
                                                const float (&kr)[KT],
@@ -64,24 +67,33 @@ __device__ __forceinline__ void stream_sources(const float4* s_keys, const int f
         const float r0 = r2 * inv;
         const float e  = __builtin_fmaf(-r0, r0, r2);
         const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
-        nzero += ok ? 0.0f : 1.0f;
+        float m = inv, mr = 1.0f;
+        if (MAG == 1) {
+            nzero += ok ? 0.0f : 1.0f;       // the r = 0 pair adds cos(0) = 1 to the cos sums: counted, removed at the end
+        } else {
+            // the r = 0 pair gets weight 0 in both sums
+            if (MAG == 0) m = ok ? 1.0f : 0.0f;
+            if (MAG == 2) m = ok ? __builtin_amdgcn_rcpf(__builtin_amdgcn_logf(r)) : 0.0f;   // v_log_f32 is log2
+            if (MAG == 3) m = ok ? __builtin_amdgcn_rsqf(r) : 0.0f;
+            mr = m * r;
+        }
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
             float ph = r * kr[t];
             if (FRACT) ph = __builtin_amdgcn_fractf(ph);
             const float s = __builtin_amdgcn_sinf(ph);
             const float c = __builtin_amdgcn_cosf(ph);
-            acc_oc[t] = __builtin_fmaf(c, inv, acc_oc[t]);
-            acc_os[t] = __builtin_fmaf(s, inv, acc_os[t]);
-            acc_c[t] += c;
-            acc_s[t] += s;
+            acc_oc[t] = __builtin_fmaf(c, m, acc_oc[t]);
+            acc_os[t] = __builtin_fmaf(s, m, acc_os[t]);
+            if (MAG == 1) { acc_c[t] += c; acc_s[t] += s; }
+            else          { acc_c[t] = __builtin_fmaf(c, mr, acc_c[t]); acc_s[t] = __builtin_fmaf(s, mr, acc_s[t]); }
         }
     }
 }
 
 // Everything after the prologue, for one choice of FRACT: the running sums live only inside this
 // function, so the two instantiations a kernel holds never have their accumulators alive together.
-template <int KT, bool SPLIT, bool FRACT>
+template <int KT, bool SPLIT, bool FRACT, int MAG>
 __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_red,
                                         const float* __restrict__ cz, const uint8_t* __restrict__ mz, const int layout,
                                         float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
@@ -123,8 +135,8 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
             if (!wave_active) continue;
 
             // -- stream the staged sources --
-            if (SPLIT) stream_sources<KT, FRACT>(s_keys, wave, WE_WAVES, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
-            else       stream_sources<KT, FRACT>(s_keys, 0, 1, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
+            if (SPLIT) stream_sources<KT, FRACT, MAG>(s_keys, wave, WE_WAVES, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
+            else       stream_sources<KT, FRACT, MAG>(s_keys, 0, 1, nk, xi, yi, zi, kr, acc_oc, acc_os, acc_c, acc_s, nzero);
         }
     }
 
@@ -197,7 +209,7 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
 //        end.  Four times as many workgroups for the same KT, still no atomics, still deterministic.
 // fract_mode  0: a workgroup reduces the phase explicitly (v_fract) only if some phase of its waves can
 //        leave +-WE_MAX_REV revolutions; 1: always; -1: never (a measuring aid, valid only for bounded phases)
-template <int KT, bool SPLIT>
+template <int KT, bool SPLIT, int MAG>
 __global__ __launch_bounds__(WE_THREADS)
 void we_fwd_kernel(const float* __restrict__ coords, const int layout,
                    const float* __restrict__ wavenumbers,
@@ -286,10 +298,10 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     }
     const bool use_fract = fract_mode > 0 || (fract_mode == 0 && !wg_safe);
     if (use_fract)
-        we_body<KT, SPLIT, true>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
+        we_body<KT, SPLIT, true, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
                                  i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
     else
-        we_body<KT, SPLIT, false>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
+        we_body<KT, SPLIT, false, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
                                   i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
 }
 
@@ -310,14 +322,14 @@ const WeVariant kVariants[] = {
 };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
-template <int KT, bool SPLIT>
+template <int KT, bool SPLIT, int MAG = 1>
 int launch(const float* coords, int layout, const float* wn, const uint8_t* mask,
            float* out, float* cs, float* ss, int Z, int N, int K, int fract, hipStream_t st)
 {
     const int iblocks = (N + 63) / 64;
     const int ktiles  = SPLIT ? (K + KT - 1) / KT : (K + KT * WE_WAVES - 1) / (KT * WE_WAVES);
     dim3 grid(iblocks, ktiles, Z);
-    hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT>), grid, dim3(WE_THREADS), 0, st,
+    hipLaunchKernelGGL((we_fwd_kernel<KT, SPLIT, MAG>), grid, dim3(WE_THREADS), 0, st,
                        coords, layout, wn, mask, out, cs, ss, N, K, fract);
     return (int)hipGetLastError();
 }
@@ -387,4 +399,37 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
         default: return WE_GO(8);
     }
 #undef WE_GO
+}
+
+namespace {
+template <int MAG>
+int launch_mag(bool split, const float* coords, int layout, const float* wn, const uint8_t* mask,
+               float* out, float* cs, float* ss, int Z, int N, int K, hipStream_t st)
+{
+    return split ? launch<8, true, MAG>(coords, layout, wn, mask, out, cs, ss, Z, N, K, 0, st)
+                 : launch<16, false, MAG>(coords, layout, wn, mask, out, cs, ss, Z, N, K, 0, st);
+}
+}  // namespace
+
+extern "C" int proteus_we_legacy_fwd(const float* coords, int coords_layout,
+                                     const float* wavenumbers, const uint8_t* mask,
+                                     float* out, float* cos_sums, float* sin_sums,
+                                     int Z, int N, int K, int magnitude_type, void* stream)
+{
+    if (magnitude_type < 0 || magnitude_type > 3) return PROTEUS_ERR_UNSUPPORTED;
+    if (magnitude_type == 1)
+        return proteus_we_fwd(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 0, stream);
+    const int rc = proteus_we_fwd_check(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 0);
+    if (rc != PROTEUS_OK) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // two tilings only for the rarely used weights: 16 wavenumbers per wave, or, while that leaves SIMDs
+    // idle, 8 per workgroup with the sources split over its four waves
+    const long iblocks = ((long)N + 63) / 64 * Z;
+    const long nwaves  = iblocks * (((long)K + 63) / 64) * WE_WAVES;
+    const bool split   = nwaves < 2048 && N >= 4 * 64;
+    switch (magnitude_type) {
+        case 0:  return launch_mag<0>(split, coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, st);
+        case 2:  return launch_mag<2>(split, coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, st);
+        default: return launch_mag<3>(split, coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, st);
+    }
 }

@@ -13,8 +13,11 @@ from . import _lib
 from .cb_utils import get_coords
 
 
-def we_forward(coords, wavenumbers, mask=None, tuning: int = 0):
+def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: int = 1):
     """out, cos_sums, sin_sums = we_forward(coords [Z,N,3], wavenumbers [K], mask [Z,N] bool | None).
+
+    magnitude_type: the weight of a source at distance r, 0: 1, 1: 1/r (default), 2: 1/log2(r),
+    3: 1/sqrt(r) (isotropic/cuda/wf_embedding_kernel.cu:192-206); the sums carry the weight times r.
 
     mask: True = padded.  Unlike the reference wrapper (which crashes on
     mask=None at isotropic/cuda/wf_embedding.py:29), None means "nothing padded".
@@ -46,10 +49,16 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0):
         return out, cos_sums, sin_sums
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
-                                None if m is None else m.data_ptr(),
-                                out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
-                                Z, N, K, int(tuning), stream)
+        if magnitude_type == 1:
+            rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
+                                    None if m is None else m.data_ptr(),
+                                    out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
+                                    Z, N, K, int(tuning), stream)
+        else:
+            rc = lib.proteus_we_legacy_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
+                                           None if m is None else m.data_ptr(),
+                                           out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
+                                           Z, N, K, int(magnitude_type), stream)
     _lib.check(rc, "proteus_we_fwd")
     return out, cos_sums, sin_sums
 
@@ -63,12 +72,9 @@ class _wf_embedding(torch.autograd.Function):
     def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask):
         if magnitude_type not in (0, 1, 2, 3):
             raise AssertionError("magnitude_type must be one of 0, 1, 2, 3")
-        if magnitude_type != 1:
-            raise NotImplementedError("only magnitude_type=1 (1/|R|) is implemented; it is the only value "
-                                      "the WaveFunctionEmbedding module passes")
         if dropout_p != 0.0:
             raise NotImplementedError("dropout_p != 0 is not implemented; the module always passes 0.0")
-        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask)
+        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type)
         ctx.save_for_backward(cos_sums, sin_sums)
         ctx.wn_dtype = wavenumbers.dtype
         return out

@@ -136,10 +136,13 @@ def test_operator_argument_errors_match_the_reference_surface():
         pa.we_forward(torch.randn(1, 8, 2), torch.rand(4))
     with pytest.raises(AssertionError):
         pa.wf_embedding(coords, torch.rand(4), magnitude_type=5)
-    with pytest.raises(NotImplementedError):
-        pa.wf_embedding(coords, torch.rand(4), magnitude_type=0)
+    with pytest.raises(_lib.ProteusError):
+        pa.wf_embedding(coords, torch.rand(4), magnitude_type=0)      # exists, but not on the CPU
     with pytest.raises(NotImplementedError):
         pa.wf_embedding(coords, torch.rand(4), dropout_p=0.1)
+    lib = _lib.load()
+    assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, 0x1000, 0x1000, 0x1000, 1, 8, 4, 4, None) == -7
+    assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, None, 0x1000, 0x1000, 1, 8, 4, 2, None) == -1
     Q = torch.randn(1, 2, 8, 64)
     with pytest.raises(AssertionError):
         pa.geo_attn(Q, Q[:, :, :4], Q, coords, torch.ones(2))

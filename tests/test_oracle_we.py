@@ -202,3 +202,39 @@ def test_row_subset_equals_full():
     t = torch_oracle.we_torch(torch.from_numpy(coords), torch.from_numpy(wn), torch.from_numpy(mask), rows=rows.tolist())
     for f, s in zip(full, t):
         assert np.abs(f[:, rows] - s.numpy()).max() < 1e-4
+
+
+@pytest.mark.parametrize("mag_type", [0, 2, 3])
+def test_other_source_weights(mag_type):
+    # two tokens 5 apart: closed form; then, on a random case, the identity the backward rests on for every
+    # weight (sums = wavenumber derivative of the embedding), and agreement with the dense statement of
+    # tests/wf_embed/wf_embed.py:108-116 written with torch
+    weight = {0: lambda d: 1.0, 2: lambda d: 1 / math.log2(d), 3: lambda d: 1 / math.sqrt(d)}[mag_type]
+    coords = np.array([[[0, 0, 0], [3, 4, 0]]], np.float32)
+    wn = np.array([0.7], np.float32)
+    out, cs, ss = c_oracle.we(coords, wn, mag_type=mag_type)
+    kk = float(wn[0])
+    assert out[0, 0, 0] == pytest.approx(weight(5.0) * math.cos(5 * kk), abs=1e-12)
+    assert out[0, 1, 1] == pytest.approx(weight(5.0) * math.sin(5 * kk), abs=1e-12)
+    assert cs[0, 0, 0] == pytest.approx(5 * weight(5.0) * math.cos(5 * kk), abs=1e-12)
+    assert ss[0, 1, 0] == pytest.approx(5 * weight(5.0) * math.sin(5 * kk), abs=1e-12)
+
+    coords, wn, mask = _random_case(20 + mag_type, Z=2, N=18, K=3)
+    coords = coords * 2 + 0.0                     # keeps distances away from 1, where 1/log2 has its pole
+    wn = (np.round((np.abs(wn) + 0.2) * 64) / 64).astype(np.float32)
+    out, cs, ss = c_oracle.we(coords, wn, mask, mag_type=mag_type)
+    h = np.float32(2.0 ** -14)
+    fd = (c_oracle.we(coords, wn + h, mask, mag_type=mag_type)[0] - c_oracle.we(coords, wn - h, mask, mag_type=mag_type)[0]) / (2 * float(h))
+    scale = max(1.0, np.abs(cs).max())
+    assert np.abs(fd[..., 0::2] + ss).max() < 1e-5 * scale
+    assert np.abs(fd[..., 1::2] - cs).max() < 1e-5 * scale
+
+    c = torch.from_numpy(coords).double()
+    d = torch.sqrt(((c[:, :, None] - c[:, None]) ** 2).sum(-1))
+    m = torch.from_numpy(mask)
+    bad = m[:, :, None] | m[:, None, :] | (d == 0)
+    dd = torch.where(bad, torch.full_like(d, float("inf")), d)
+    mag = {0: torch.where(bad, torch.zeros_like(d), torch.ones_like(d)), 2: 1 / torch.log2(dd), 3: 1 / torch.sqrt(dd)}[mag_type]
+    ph = d[..., None] * torch.from_numpy(wn).double()
+    feats = torch.stack([(mag[..., None] * torch.cos(ph)).sum(2), (mag[..., None] * torch.sin(ph)).sum(2)], -1).flatten(2)
+    np.testing.assert_allclose(out, feats.numpy(), rtol=0, atol=1e-11)

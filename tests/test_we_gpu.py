@@ -283,3 +283,28 @@ def test_hardware_sincos_and_sqrt_error(gpu):
     torch.cuda.synchronize()
     ref = np.sqrt(r2.double().numpy())
     assert (np.abs(q.cpu().numpy() - ref) / np.maximum(ref, 1e-30)).max() < 1.2e-7
+
+
+@pytest.mark.parametrize("mag_type", [0, 2, 3])
+@pytest.mark.parametrize("N,Z,K", [(300, 2, 40), (2048, 1, 256)])
+def test_other_source_weights(gpu, mag_type, N, Z, K):
+    # the reference's magnitude_type 0 / 2 / 3 (isotropic/cuda/wf_embedding_kernel.cu:192-206), both tilings
+    coords, _ = synth.we_inputs(N, seed=40 + mag_type, batch=Z)
+    wn = synth.wavenumbers(2 * K)
+    mask = torch.rand(Z, N, generator=torch.Generator().manual_seed(N)) < 0.2
+    got = pa.we_forward(coords.to(gpu), wn.to(gpu), mask.to(gpu), magnitude_type=mag_type)
+    rows = None if N <= 512 else np.arange(0, N, 37)
+    ref = c_oracle.we(coords.numpy(), wn.numpy(), mask.numpy(), rows=rows, mag_type=mag_type)
+    sel = slice(None) if rows is None else rows
+    for g, r, name in zip(got, ref, ("out", "cos_sums", "sin_sums")):
+        g = g.cpu().numpy()
+        assert (g[mask.numpy()] == 0).all()
+        assert rel_l2(g[:, sel], r) <= REL_L2_TOL, f"magnitude_type {mag_type} {name}: {rel_l2(g[:, sel], r):.3e}"
+    # and through the autograd function: the backward consumes these sums unchanged
+    w = wn.to(gpu).requires_grad_(True)
+    out = pa.wf_embedding(coords.to(gpu), w, magnitude_type=mag_type, mask=mask.to(gpu))
+    out.sum().backward()
+    dk = torch_oracle.we_backward_torch(torch.ones(Z, N if rows is None else len(rows), 2 * K, dtype=torch.float64),
+                                        torch.from_numpy(ref[1]), torch.from_numpy(ref[2]))
+    if rows is None:
+        assert rel_l2(w.grad.cpu().numpy(), dk.numpy()) <= REL_L2_TOL
