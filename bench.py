@@ -24,8 +24,10 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0      # dense bf16 matrix
 H100_REFERENCE_GPW = 6.87194767e10 / 0.386 / 1e9   # README.md:34: 386 ms at this exact shape on an H100
 
 # HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), bytes
-WE_TRAFFIC_BYTES = None
-ATTN_TRAFFIC_BYTES = None
+# WE: FETCH_SIZE 4370.5 KiB x 2.0 (calibration factor of that counter) + WRITE_SIZE 82271.9 KiB x 1.0
+WE_TRAFFIC_BYTES = int((4370.5 * 2.0 + 82271.9) * 1024)
+# attention: FETCH_SIZE (42510.3 + 830.6) KiB x 2.0 over its two launches + WRITE_SIZE 33280.0 KiB x 1.0
+ATTN_TRAFFIC_BYTES = int(((42510.3 + 830.6) * 2.0 + 33280.0) * 1024)
 
 
 def median(xs):
@@ -35,10 +37,12 @@ def median(xs):
 
 def probe_rates(lib, torch, dev):
     """Measured lane-op rates (lane-ops/s) of the instructions the WE inner loop issues."""
-    names = ["fma", "mul", "add", "sin", "cos", "exp2", "rsq", "fract"]
+    # scalar-operand forms (ops 0-2), transcendentals, and the vector-operand forms of the accumulations
+    names = {0: "fma_s", 1: "mul_s", 2: "add_s", 3: "sin", 4: "cos", 5: "exp2", 6: "rsq", 7: "fract",
+             20: "fmac_v", 21: "add_v"}
     sink = torch.empty(2048 * 256, device=dev)
     rates = {}
-    for op, name in enumerate(names):
+    for op, name in names.items():
         blocks, iters = 2048, 1000
         lib.proteus_probe_valu_rate(op, blocks, iters, sink.data_ptr(), None)
         torch.cuda.synchronize()
@@ -58,6 +62,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-attn", action="store_true", help="skip the geometric attention leg")
+    ap.add_argument("--no-aniso", action="store_true", help="skip the anisotropic WE leg")
     ap.add_argument("--no-encoder", action="store_true", help="skip the encoder-forward leg (BASELINE.json configs[3])")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--we-tuning", type=int, default=0)
@@ -113,17 +118,19 @@ def main():
     value = W * args.steps / elapsed / 1e9            # Gpair*wavenumber/s, whole job
 
     rates = probe_rates(lib, torch, dev)
-    r_valu = (rates["fma"] + rates["mul"] + rates["add"]) / 3
+    # per unit: the phase product (scalar operand), v_sin, v_cos, two v_fmac and two v_add on vector operands
     r_trans = (rates["sin"] + rates["cos"]) / 2
-    t_model_ms = W * (5.0 / r_valu + 2.0 / r_trans) * 1e3       # 5 fp32 VALU + 2 transcendental lane-ops per unit
+    t_model_ms = W * (1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / rates["add_v"] + 2.0 / r_trans) * 1e3
     achieved_tflops = 9.0 * W / (avg_kernel_ms * 1e-3) / 1e12   # 9 flop per unit, FMA counted as 2
     roofline = {
         "kernel": "we_fwd_kernel", "bound": "valu", "achieved": achieved_tflops, "peak": PEAK_FP32_VECTOR_TFLOPS,
         "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_FP32_VECTOR_TFLOPS, "traffic": WE_TRAFFIC_BYTES,
         "kernel_ms": avg_kernel_ms,
         "issue_model": {
-            "lane_ops_per_unit": {"valu_fp32": 5, "transcendental": 2},
-            "measured_rate_valu_lane_ops_per_s": r_valu, "measured_rate_trans_lane_ops_per_s": r_trans,
+            "lane_ops_per_unit": {"mul_scalar_operand": 1, "fmac_vector_operands": 2, "add_vector_operands": 2,
+                                  "transcendental": 2},
+            "measured_lane_ops_per_s": {"mul_scalar_operand": rates["mul_s"], "fmac_vector_operands": rates["fmac_v"],
+                                        "add_vector_operands": rates["add_v"], "transcendental": r_trans},
             "model_ms": t_model_ms, "frac": t_model_ms / avg_kernel_ms,
         },
     }
@@ -140,6 +147,41 @@ def main():
                    "Z": Z, "N": N, "K": K, "we_variant": _lib.we_variants()[args.we_tuning]},
         "roofline": roofline,
     }
+
+    # ---------------- anisotropic (C-beta scaled) WE forward, same shape and chain ----------------
+    if not args.no_aniso:
+        g = torch.Generator().manual_seed(2)
+        cbv = torch.randn(Z, N, 3, generator=g)
+        cbv = (cbv / cbv.norm(dim=-1, keepdim=True)).to(dev).contiguous()
+        cbm = (0.5 + 2.0 * torch.rand(K, generator=g)).to(dev)
+        ao = [torch.empty(Z, N, 2 * K, device=dev) for _ in range(3)]
+
+        def aniso_step():
+            rc = lib.proteus_we_aniso_fwd(c.data_ptr(), cbv.data_ptr(), _lib.COORDS_AOS, cbm.data_ptr(), w.data_ptr(), None,
+                                          ao[0].data_ptr(), ao[1].data_ptr(), ao[2].data_ptr(), Z, N, K, 0, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_we_aniso_fwd")
+        for _ in range(2):
+            aniso_step()
+        torch.cuda.synchronize()
+        n_it = max(5, args.steps // 2)
+        xev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_it)]
+        for e0, e1 in xev:
+            e0.record()
+            aniso_step()
+            e1.record()
+        torch.cuda.synchronize()
+        x_ms = sum(e0.elapsed_time(e1) for e0, e1 in xev) / n_it
+        # per unit: 2 scalar-operand phase ops, v_fract, 4 v_fmac + 2 v_add on vector operands, v_sin, v_cos
+        x_model_ms = W * (2.0 / rates["mul_s"] + 1.0 / rates["fract"] + 4.0 / rates["fmac_v"] + 2.0 / rates["add_v"]
+                          + 2.0 / r_trans) * 1e3
+        result["we_aniso"] = {
+            "workload": "anisotropic (C-beta scaled) WE forward, out + d_cb + d_k, B=1 N=16384 256 wavenumbers, same chain, random unit C-beta vectors",
+            "ms": x_ms, "gpair_wavenumber_per_s": W / (x_ms * 1e-3) / 1e9, "dtype": "f32",
+            "issue_model": {"lane_ops_per_unit": {"scalar_operand": 2, "fract": 1, "fmac_vector_operands": 4,
+                                                  "add_vector_operands": 2, "transcendental": 2},
+                            "model_ms": x_model_ms, "frac": x_model_ms / x_ms},
+        }
 
     # ---------------- geometric attention forward, N=16384, H=8, d=64 (configs[4]) ----------------
     if not args.no_attn:

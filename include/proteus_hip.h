@@ -213,7 +213,22 @@ const char* proteus_geo_attn_variant_name(int tuning);
  * launch; lane-ops issued = blocks*256*iters*64.  No counterpart in the
  * reference.
  *   op: 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_sin_f32, 4 v_cos_f32,
- *       5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32
+ *       5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32;
+ *       8, 9, 10: one stream mixing 16 v_sin_f32 chains with 16, 32, 48 v_fma_f32
+ *       chains (lane-ops issued = blocks*256*iters*(16 + 16|32|48)): whether the
+ *       transcendental and the ordinary fp32 pipelines overlap;
+ *       11, 12, 13: the same with a fixed program order, every v_sin_f32 followed
+ *       by 1, 2, 3 v_fma_f32 (lane-ops = blocks*256*iters*16*(1 + 1|2|3));
+ *       14: blocks/2 workgroups of 8 waves, four running 64 v_sin_f32 chains and four 64 v_fma_f32 chains
+ *       (overlap across waves of one SIMD);
+ *       15, 17: the embedding kernel's inner step on register data, 8 and 32
+ *       wavenumbers per step (7 instructions each, two of them transcendental);
+ *       16, 18: the same with the two transcendentals replaced by multiplies;
+ *       19..22: 64 chains with vector-register operands only: x = fma(x,u,v),
+ *       x = fma(u,v,x), x += u, x *= u (ops 0..2 feed scalar-register operands);
+ *       23..26: blocks/2 workgroups of 8 waves, 16 links per lane and round of
+ *       v_mfma_f32_4x4x1_16B_f32 alone, v_sin_f32 alone, both in one stream, and
+ *       four waves of each kind (matrix pipeline beside the transcendental one)
  */
 int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
 

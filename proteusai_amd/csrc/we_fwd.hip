@@ -35,7 +35,17 @@ namespace {
 constexpr int WE_WAVES   = 4;
 constexpr int WE_THREADS = WE_WAVES * 64;
 constexpr int WE_JB      = 256;   // sources staged per LDS block (one per thread)
-constexpr float WE_MAX_REV = 250.0f;   // v_sin_f32 / v_cos_f32 accept |x| <= 256 revolutions; keep a margin
+constexpr float WE_MAX_REV = 250.0f;
+
+// Wavenumbers per phase batch of the inner loop (0: leave the order to the compiler).  On gfx950 a
+// vector instruction whose operands are all vector registers issues in about 2.4 clocks per wave once a
+// SIMD holds three or more waves, one with a scalar-register operand in 4, a transcendental in 8; an
+// ordinary instruction placed between two transcendentals of the same wave costs 4 whatever its operands
+// (measured with proteus_probe_valu_rate).  So the loop does the scalar-operand phase products of a batch
+// first, then its sines and cosines, then its accumulations, which then run at the fast rate.
+#ifndef WE_BATCH
+#define WE_BATCH 16
+#endif   // v_sin_f32 / v_cos_f32 accept |x| <= 256 revolutions; keep a margin
 
 __device__ __forceinline__ float sgpr(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
@@ -77,16 +87,34 @@ __device__ __forceinline__ void stream_sources(const float4* s_keys, const int f
             if (MAG == 3) m = ok ? __builtin_amdgcn_rsqf(r) : 0.0f;
             mr = m * r;
         }
+        // The wavenumbers are taken in batches and each batch in three phases (phases, then sines and
+        // cosines, then the accumulations), kept apart by scheduling barriers: see WE_BATCH.
+        constexpr int B = (WE_BATCH > 0 && WE_BATCH < KT) ? WE_BATCH : KT;
 #pragma unroll
-        for (int t = 0; t < KT; ++t) {
-            float ph = r * kr[t];
-            if (FRACT) ph = __builtin_amdgcn_fractf(ph);
-            const float s = __builtin_amdgcn_sinf(ph);
-            const float c = __builtin_amdgcn_cosf(ph);
-            acc_oc[t] = __builtin_fmaf(c, m, acc_oc[t]);
-            acc_os[t] = __builtin_fmaf(s, m, acc_os[t]);
-            if (MAG == 1) { acc_c[t] += c; acc_s[t] += s; }
-            else          { acc_c[t] = __builtin_fmaf(c, mr, acc_c[t]); acc_s[t] = __builtin_fmaf(s, mr, acc_s[t]); }
+        for (int t0 = 0; t0 < KT; t0 += B) {
+            float sn[B], cs[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+                float ph = r * kr[t0 + u];
+                if (FRACT) ph = __builtin_amdgcn_fractf(ph);
+                sn[u] = ph;
+            }
+            if (WE_BATCH > 0) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+                cs[u] = __builtin_amdgcn_cosf(sn[u]);
+                sn[u] = __builtin_amdgcn_sinf(sn[u]);
+            }
+            if (WE_BATCH > 0) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+                const int t = t0 + u;
+                acc_oc[t] = __builtin_fmaf(cs[u], m, acc_oc[t]);
+                acc_os[t] = __builtin_fmaf(sn[u], m, acc_os[t]);
+                if (MAG == 1) { acc_c[t] += cs[u]; acc_s[t] += sn[u]; }
+                else          { acc_c[t] = __builtin_fmaf(cs[u], mr, acc_c[t]); acc_s[t] = __builtin_fmaf(sn[u], mr, acc_s[t]); }
+            }
+            if (WE_BATCH > 0) __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -141,29 +169,30 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
     }
 
     if (SPLIT) {
-        // ---- the four waves' partial sums meet in LDS; wave 0 writes the rows ----
-        __syncthreads();
-        if (wave > 0) {
-            float* r = s_red + (size_t)(wave - 1) * (4 * KT + 1) * 64 + lane;
+        // ---- the four waves' partial sums meet in LDS, one wave at a time; wave 0 writes the rows ----
+        float* q = s_red + lane;
+#pragma unroll 1
+        for (int w = 1; w < WE_WAVES; ++w) {
+            __syncthreads();
+            if (wave == w) {
 #pragma unroll
-            for (int t = 0; t < KT; ++t) {
-                r[(4 * t + 0) * 64] = acc_oc[t]; r[(4 * t + 1) * 64] = acc_os[t];
-                r[(4 * t + 2) * 64] = acc_c[t];  r[(4 * t + 3) * 64] = acc_s[t];
+                for (int t = 0; t < KT; ++t) {
+                    q[(4 * t + 0) * 64] = acc_oc[t]; q[(4 * t + 1) * 64] = acc_os[t];
+                    q[(4 * t + 2) * 64] = acc_c[t];  q[(4 * t + 3) * 64] = acc_s[t];
+                }
+                q[4 * KT * 64] = nzero;
             }
-            r[4 * KT * 64] = nzero;
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int t = 0; t < KT; ++t) {
+                    acc_oc[t] += q[(4 * t + 0) * 64]; acc_os[t] += q[(4 * t + 1) * 64];
+                    acc_c[t]  += q[(4 * t + 2) * 64]; acc_s[t]  += q[(4 * t + 3) * 64];
+                }
+                nzero += q[4 * KT * 64];
+            }
         }
-        __syncthreads();
         if (wave > 0) return;
-#pragma unroll
-        for (int w = 0; w < WE_WAVES - 1; ++w) {
-            const float* r = s_red + (size_t)w * (4 * KT + 1) * 64 + lane;
-#pragma unroll
-            for (int t = 0; t < KT; ++t) {
-                acc_oc[t] += r[(4 * t + 0) * 64]; acc_os[t] += r[(4 * t + 1) * 64];
-                acc_c[t]  += r[(4 * t + 2) * 64]; acc_s[t]  += r[(4 * t + 3) * 64];
-            }
-            nzero += r[4 * KT * 64];
-        }
     }
 
     if (!wave_active || !i_in) return;
@@ -210,7 +239,7 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
 // fract_mode  0: a workgroup reduces the phase explicitly (v_fract) only if some phase of its waves can
 //        leave +-WE_MAX_REV revolutions; 1: always; -1: never (a measuring aid, valid only for bounded phases)
 template <int KT, bool SPLIT, int MAG>
-__global__ __launch_bounds__(WE_THREADS)
+__global__ __launch_bounds__(WE_THREADS, (KT == 32 && SPLIT) ? 3 : 1)
 void we_fwd_kernel(const float* __restrict__ coords, const int layout,
                    const float* __restrict__ wavenumbers,
                    const uint8_t* __restrict__ mask,
@@ -220,7 +249,7 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     __shared__ float4 s_keys[WE_JB + WE_WAVES];   // padding: the stream loop reads one step ahead
     __shared__ int    s_wcount[WE_WAVES];
     __shared__ float  s_box[WE_WAVES][6];
-    __shared__ float  s_red[SPLIT ? (WE_WAVES - 1) * (4 * KT + 1) * 64 : 1];
+    __shared__ float  s_red[SPLIT ? (4 * KT + 1) * 64 : 1];
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -317,6 +346,7 @@ const WeVariant kVariants[] = {
     {"kt8", 8, false, 0},
     {"kt16_split", 16, true, 0},
     {"kt8_split", 8, true, 0},
+    {"kt32_split", 32, true, 0},
     {"kt32_fract", 32, false, 1},
     {"kt32_nofract_unchecked", 32, false, -1},
 };
@@ -371,30 +401,37 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
     const int fract = kVariants[tuning].fract;
     const long iblocks = ((long)N + 63) / 64 * Z;
     if (tuning == 0) {
-        // Pick the (wavenumber tile, source split) pair with the least estimated issue time:
-        // instructions per wave x rounds of 1024 waves, with a penalty when a SIMD would hold a
-        // single wave (nothing to cover its LDS and transcendental latencies).  Ties keep the
-        // earlier candidate (wider tile, no split).
-        static const int cand_kt[5]    = {32, 16, 8, 16, 8};
-        static const int cand_split[5] = {0, 0, 0, 1, 1};
+        // Pick the (wavenumber tile, source split) pair with the least estimated time.  Per source a wave
+        // issues KT x (1 scalar-operand product, 2 transcendentals, 4 accumulations) + about 15 ordinary
+        // instructions and a v_rsq; what an instruction costs depends on how many waves share the SIMD
+        // (clocks per wave instruction, measured: vector-operand 5.8 / 2.9 / 2.5, scalar-operand
+        // 4.8 / 4.15 / 4.0, transcendental 10.3 / 9.0 / 8.3 with 1 / 2 / 3+ waves).  `occ` is what the
+        // kernel's registers allow.  Ties keep the earlier candidate.
+        static const int cand_kt[6]    = {32, 32, 16, 16, 8, 8};
+        static const int cand_split[6] = {1, 0, 1, 0, 1, 0};
+        static const int cand_occ[6]   = {3, 2, 4, 4, 8, 8};
         double best = 1e300;
-        for (int c = 0; c < 5; ++c) {
+        for (int c = 0; c < 6; ++c) {
             const int  ckt = cand_kt[c];
             const bool csp = cand_split[c] != 0;
             if (csp && N < 4 * 64) continue;
             const long ktiles = ((long)K + ckt - 1) / ckt;
             const long nwaves = csp ? iblocks * ktiles * WE_WAVES : iblocks * ((ktiles + WE_WAVES - 1) / WE_WAVES) * WE_WAVES;
             const double keys = csp ? (double)N / WE_WAVES : (double)N;
-            const double rounds = (double)((nwaves + 1023) / 1024);
-            double est = rounds * keys * (8.0 * ckt + 17.0);
-            if (nwaves < 2048) est *= 1.25;
+            const double q    = (double)nwaves / 1024.0;                 // waves per SIMD over the whole launch
+            const int    w    = q > cand_occ[c] ? cand_occ[c] : (q <= 1.0 ? 1 : (int)(q + 0.999));
+            const double cv = w <= 1 ? 5.8 : (w == 2 ? 2.9 : 2.5);
+            const double cs = w <= 1 ? 4.8 : (w == 2 ? 4.15 : 4.0);
+            const double ct = w <= 1 ? 10.3 : (w == 2 ? 9.0 : 8.3);
+            const double per_wave = keys * (ckt * (cs + 2.0 * ct + 4.0 * cv) + 15.0 * cv + ct + 30.0);
+            const double est = (q > w ? q : (double)w) * per_wave;
             if (est < best * 0.999) { best = est; kt = ckt; split = csp; }
         }
     }
 #define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st) \
                           : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st))
     switch (kt) {
-        case 32: return launch<32, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st);
+        case 32: return WE_GO(32);
         case 16: return WE_GO(16);
         default: return WE_GO(8);
     }

@@ -120,7 +120,10 @@ def test_masks(gpu):
 def test_coincident_points_and_reference_sentinel(gpu):
     coords, wn = synth.we_inputs(90, seed=6, d_model=32)
     coords[0, 40] = coords[0, 12]                     # coincident pair -> dropped like the self pair
-    coords[0, 50, 0] = 12345.0                        # the reference's in-band mask value is an ordinary coordinate here
+    # the reference's in-band mask value is an ordinary coordinate here: move the chain so that token 50 sits
+    # at x == 12345.0 exactly (a lone far-away point would only test fp32's phase rounding at thousands of turns)
+    coords[0, :, 0] += 12345.0 - coords[0, 50, 0]
+    coords[0, 50, 0] = 12345.0
     check(run_gpu(gpu, coords, wn), coords, wn, what="coincident")
 
 
