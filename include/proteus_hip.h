@@ -228,7 +228,9 @@ const char* proteus_geo_attn_variant_name(int tuning);
  *       x = fma(u,v,x), x += u, x *= u (ops 0..2 feed scalar-register operands);
  *       23..26: blocks/2 workgroups of 8 waves, 16 links per lane and round of
  *       v_mfma_f32_4x4x1_16B_f32 alone, v_sin_f32 alone, both in one stream, and
- *       four waves of each kind (matrix pipeline beside the transcendental one)
+ *       four waves of each kind (matrix pipeline beside the transcendental one);
+ *       27..30: per link four v_mfma_f32_32x32x16_bf16 alone, 32 v_fmac_f32 alone,
+ *       both in one stream, and the MFMAs with 32 v_exp_f32 in one stream
  */
 int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
 

@@ -186,6 +186,49 @@ void mfma_sin_mix_kernel(float* sink, int iters, float a, float b) {
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// The attention kernel's matrix instruction beside ordinary vector work.  Per link: MODE 0: four independent
+// v_mfma_f32_32x32x16_bf16; 1: 32 v_fmac_f32 on vector operands; 2: both in one instruction stream (eight
+// v_fmac_f32 after each MFMA); 3: as 2 with v_exp_f32 chains in place of the v_fmac_f32.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+template <int MODE>
+__global__ __launch_bounds__(256)
+void mfma_valu_mix_kernel(float* sink, int iters, float a, float b) {
+    f32x16 d[4];
+    float x[32];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) d[c][e] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 32; ++c) x[c] = 0.001f * (float)(threadIdx.x + c) + 0.25f;
+    float u = 1e-3f * a + 1e-9f * (float)threadIdx.x, v = b + 1e-12f * (float)threadIdx.x;
+    bf16x8_t pa, pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { pa[e] = (__bf16)(0.01f * (float)(threadIdx.x & 7)); pb[e] = (__bf16)(0.02f * (float)e); }
+#pragma unroll 1
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (MODE != 1) d[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, pb, d[c], 0, 0, 0);
+#pragma unroll
+            for (int f = 0; f < 8; ++f) {
+                if (MODE == 1 || MODE == 2) x[8 * c + f] = __builtin_fmaf(u, v, x[8 * c + f]);
+                if (MODE == 3) x[8 * c + f] = __builtin_amdgcn_exp2f(x[8 * c + f]);
+            }
+        }
+        asm volatile("" : "+v"(u), "+v"(v));
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 32; ++c) s += x[c];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += d[c][e];
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // The same mix in a fixed program order: every v_sin_f32 is followed by NF_PER ordinary instructions
 // before the next one (the compiler, left alone, tends to group the transcendentals).
 template <int NF_PER>
@@ -253,13 +296,17 @@ extern "C" const char* proteus_strerror(int code) {
 extern "C" int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;
     if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return PROTEUS_ERR_BAD_SHAPE;
-    if (op < 0 || op > 26) return PROTEUS_ERR_BAD_TUNING;
+    if (op < 0 || op > 30) return PROTEUS_ERR_BAD_TUNING;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // a, b chosen so that the chains stay finite and are not constant-folded
     const float a = 0.999999f, b = 1e-7f;
 #define GO(OP_) hipLaunchKernelGGL((valu_rate_kernel<OP_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
 #define MIX(NT_, NF_) hipLaunchKernelGGL((valu_mix_kernel<NT_, NF_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
     switch (op) {
+        case 27: hipLaunchKernelGGL((mfma_valu_mix_kernel<0>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
+        case 28: hipLaunchKernelGGL((mfma_valu_mix_kernel<1>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
+        case 29: hipLaunchKernelGGL((mfma_valu_mix_kernel<2>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
+        case 30: hipLaunchKernelGGL((mfma_valu_mix_kernel<3>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
         case 23: hipLaunchKernelGGL((mfma_sin_mix_kernel<0>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
         case 24: hipLaunchKernelGGL((mfma_sin_mix_kernel<1>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
         case 25: hipLaunchKernelGGL((mfma_sin_mix_kernel<2>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
