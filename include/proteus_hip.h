@@ -230,7 +230,10 @@ const char* proteus_geo_attn_variant_name(int tuning);
  *       v_mfma_f32_4x4x1_16B_f32 alone, v_sin_f32 alone, both in one stream, and
  *       four waves of each kind (matrix pipeline beside the transcendental one);
  *       27..30: per link four v_mfma_f32_32x32x16_bf16 alone, 32 v_fmac_f32 alone,
- *       both in one stream, and the MFMAs with 32 v_exp_f32 in one stream
+ *       both in one stream, and the MFMAs with 32 v_exp_f32 in one stream;
+ *       31..33: blocks/2 workgroups of 8 waves: waves 0-3 alone (four MFMAs per
+ *       link), waves 4-7 alone (16 v_exp_f32 + 16 v_fmac_f32 per link), both kinds
+ *       together (matrix and vector work in different waves of a SIMD)
  */
 int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
 

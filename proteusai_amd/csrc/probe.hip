@@ -229,6 +229,55 @@ void mfma_valu_mix_kernel(float* sink, int iters, float a, float b) {
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// Matrix and vector work in DIFFERENT waves of one SIMD: workgroups of 8 waves, waves 0-3 run
+// v_mfma_f32_32x32x16_bf16 only (MODE 0 and 2), waves 4-7 alternate 8 v_exp_f32 with 8 v_fmac_f32 on vector
+// operands (MODE 1 and 2).  Per link: 4 MFMAs in the one kind of wave, 16 + 16 vector instructions in the other.
+template <int MODE>
+__global__ __launch_bounds__(512)
+void mfma_cross_wave_kernel(float* sink, int iters, float a, float b) {
+    float s = 0.f;
+    if (threadIdx.x < 256) {
+        if (MODE == 1) return;
+        f32x16 d[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) d[c][e] = 0.f;
+        bf16x8_t pa, pb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { pa[e] = (__bf16)(0.01f * (float)(threadIdx.x & 7)); pb[e] = (__bf16)(0.02f * (float)e); }
+#pragma unroll 1
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) d[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, pb, d[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += d[c][e];
+    } else {
+        if (MODE == 0) return;
+        float x[16], y[16];
+#pragma unroll
+        for (int c = 0; c < 16; ++c) { x[c] = 0.001f * (float)(threadIdx.x + c) - 0.75f; y[c] = 0.5f + 0.01f * (float)c; }
+        float u = 1e-3f * a + 1e-9f * (float)threadIdx.x, v = b + 1e-12f * (float)threadIdx.x;
+#pragma unroll 1
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) x[8 * h + c] = __builtin_amdgcn_exp2f(x[8 * h + c] - 1.0f);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) y[8 * h + c] = __builtin_fmaf(u, v, y[8 * h + c]);
+            }
+            asm volatile("" : "+v"(u), "+v"(v));
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) s += x[c] + y[c];
+    }
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // The same mix in a fixed program order: every v_sin_f32 is followed by NF_PER ordinary instructions
 // before the next one (the compiler, left alone, tends to group the transcendentals).
 template <int NF_PER>
@@ -296,13 +345,16 @@ extern "C" const char* proteus_strerror(int code) {
 extern "C" int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;
     if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return PROTEUS_ERR_BAD_SHAPE;
-    if (op < 0 || op > 30) return PROTEUS_ERR_BAD_TUNING;
+    if (op < 0 || op > 33) return PROTEUS_ERR_BAD_TUNING;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // a, b chosen so that the chains stay finite and are not constant-folded
     const float a = 0.999999f, b = 1e-7f;
 #define GO(OP_) hipLaunchKernelGGL((valu_rate_kernel<OP_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
 #define MIX(NT_, NF_) hipLaunchKernelGGL((valu_mix_kernel<NT_, NF_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
     switch (op) {
+        case 31: hipLaunchKernelGGL((mfma_cross_wave_kernel<0>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
+        case 32: hipLaunchKernelGGL((mfma_cross_wave_kernel<1>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
+        case 33: hipLaunchKernelGGL((mfma_cross_wave_kernel<2>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
         case 27: hipLaunchKernelGGL((mfma_valu_mix_kernel<0>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
         case 28: hipLaunchKernelGGL((mfma_valu_mix_kernel<1>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
         case 29: hipLaunchKernelGGL((mfma_valu_mix_kernel<2>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
