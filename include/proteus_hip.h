@@ -202,6 +202,37 @@ int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K, const uint
                                 int Z, int H, int N, int d_head,
                                 float min_rbf, float max_rbf, int tuning, void* stream);
 
+/*
+ * Backward of both attention forwards: dQ, dK, dV, d sigma (and d beta).
+ *
+ * Replaces the Triton launch `_attn_bwd[grid](...)` of
+ *   old/old_scripts/attn/geometric_attn.py:627-648 (kernel :262-543).
+ * The caller passes what the reference's wrapper computes around that launch (:609-660):
+ * dO cast to the operand type, D = rowsum(O * dO), the forward's L, and dQ/dK/dV/d_sigma/d_beta
+ * buffers.  beta == NULL selects the README logits (proteus_geo_attn_fwd), otherwise the
+ * logits and pair mask of proteus_geo_attn_legacy_fwd.
+ *
+ *   Q, K, V, dO   [Z,H,N,64] bf16 (raw uint16), 16-byte aligned
+ *   coords [Z,N,3] f32; sigma [H] f32; beta [H] f32 or NULL; key_pad_mask [Z,N] u8 or NULL
+ *   L, D          [Z,H,N] f32
+ *   dQ, dK, dV    [Z,H,N,64] f32, 16-byte aligned, fully overwritten (zeros at padded tokens)
+ *   d_sigma       [H] f32, ACCUMULATED into with atomic adds (as the reference does, :541-543):
+ *                 zero it first; may be NULL.  d_beta likewise (legacy logits only).
+ */
+int proteus_geo_attn_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                         const float* coords, const float* sigma, const float* beta,
+                         const uint8_t* key_pad_mask, const float* L, const float* D,
+                         float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
+                         int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream);
+
+/* Validation half of proteus_geo_attn_bwd: same checks, no HIP call. */
+int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                               const float* coords, const float* sigma, const float* beta,
+                               const uint8_t* key_pad_mask, const float* L, const float* D,
+                               const float* dQ, const float* dK, const float* dV,
+                               const float* d_sigma, const float* d_beta,
+                               int Z, int H, int N, int d_head, float min_rbf, float max_rbf);
+
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);
 

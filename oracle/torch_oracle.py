@@ -159,3 +159,29 @@ def geo_attn_legacy_torch(Q, K, V, coords, spreads, b, mask=None, min_rbf=0.0, m
     P = torch.softmax(S, dim=-1)
     P = torch.where(torch.isnan(P), torch.zeros_like(P), P)
     return torch.matmul(P, V), torch.logsumexp(S, dim=-1)
+
+
+def geo_attn_autograd_torch(Q, K, V, coords, sigma, key_padding_mask=None, betas=None, min_rbf=0.0, max_rbf=1.0,
+                            dtype=torch.float64):
+    """The dense statements above in a form torch.autograd can differentiate in Q, K, V, sigma and betas
+    (the oracle of the backward kernel: nothing of the hand-derived gradient formulas enters here).
+    betas=None: logits S*(1+rbf); otherwise the reference's S + b*rbf_norm*|S| with its pair mask.
+    Rows without any unmasked pair give O = 0 and pass no gradient."""
+    Q, K, V = Q.to(dtype), K.to(dtype), V.to(dtype)
+    coords, sigma = coords.to(dtype), sigma.to(dtype)
+    Z, H, N, d = Q.shape
+    mask = torch.zeros(Z, N, dtype=torch.bool) if key_padding_mask is None else key_padding_mask.bool()
+    S = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(d)
+    d2 = torch.sum((coords[:, :, None, :] - coords[:, None, :, :]) ** 2, dim=3)[:, None, :, :]
+    rbf = torch.exp(-d2 / (2 * sigma[None, :, None, None] ** 2))
+    am = (mask[:, None, :, None] | mask[:, None, None, :]).expand(Z, H, N, N)
+    if betas is None:
+        T = S * (1 + rbf)
+    else:
+        am = am | (rbf < min_rbf) | (rbf > max_rbf)
+        T = S + betas.to(dtype)[None, :, None, None] * ((2 * (rbf - min_rbf) / (max_rbf - min_rbf)) - 1) * torch.abs(S)
+    T = torch.where(am, torch.full_like(T, float("-inf")), T)
+    row_any = (~am).any(dim=-1, keepdim=True)
+    T = torch.where(row_any, T, torch.zeros_like(T))
+    P = torch.softmax(T, dim=-1) * row_any.to(dtype)
+    return torch.matmul(P, V)

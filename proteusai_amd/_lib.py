@@ -17,7 +17,8 @@ SYMBOLS = [
     "proteus_version", "proteus_strerror",
     "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_num_variants", "proteus_we_variant_name",
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
-    "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_num_variants",
+    "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
+    "proteus_geo_attn_bwd_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_probe_valu_rate", "proteus_probe_sincos",
 ]
@@ -64,6 +65,11 @@ def load():
     lib.proteus_geo_attn_legacy_fwd.restype = ci
     lib.proteus_geo_attn_legacy_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci,
                                                 ctypes.c_float, ctypes.c_float, ci, vp]
+    cf = ctypes.c_float
+    lib.proteus_geo_attn_bwd.restype = ci
+    lib.proteus_geo_attn_bwd.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf, vp]
+    lib.proteus_geo_attn_bwd_check.restype = ci
+    lib.proteus_geo_attn_bwd_check.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf]
     lib.proteus_geo_attn_fwd_check.restype = ci
     lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_num_variants.restype = ci

@@ -1,0 +1,359 @@
+// RBF-scaled geometric attention backward for gfx950 (MI355X): dQ, dK, dV, d sigma (and d beta).
+//
+// What it computes (reference: old/old_scripts/attn/geometric_attn.py:262-543, wrapper :609-660), with
+// S = q.k/sqrt(d), rbf = exp(-|r_i - r_j|^2/(2 sigma_h^2)) and the logits t(S, rbf) of the forward kernel:
+//     P    = exp(t - L_i)                 (L: the forward's logsumexp; 0 for a masked pair)      :453
+//     dV_j = sum_i P_ij dO_i                                                                      :459
+//     dP   = dO_i . V_j ;  dt = P (dP - D_i),  D_i = sum_d O_id dO_id                             :462-465
+//     dS   = dt * dt/dS ;  dQ_i = sum_j dS_ij K_j / sqrt(d) ;  dK_j = sum_i dS_ij Q_i / sqrt(d)   :468,500-505
+//     d sigma_h = sum dt * dt/drbf * rbf * |r_i - r_j|^2 / sigma_h^3                              :473,494-497
+//   README logits  t = S (1 + rbf):             dt/dS = 1 + rbf,              dt/drbf = S
+//   LEGACY logits  t = S + beta Rn |S|, Rn = 2 (rbf - min)/(max - min) - 1   (:448-449):
+//                  dt/dS = 1 + beta Rn sign(S), dt/drbf = 2 beta |S|/(max - min), d beta_h = sum dt Rn |S|  (:468-479)
+//
+// Two launches instead of the reference's one kernel with atomic adds into dQ (:501-503):
+//   OWN_Q = false  a wave owns 32 keys, streams the queries, accumulates dK, dV (and d sigma, d beta);
+//   OWN_Q = true   a wave owns 32 queries, streams the keys, accumulates dQ.
+// Both are the same code.  Scores are computed with the rows of the streamed ("other") tokens in the
+// accumulator rows and the wave's own token in the accumulator column (lane % 32), so a lane owns one own
+// token: S = other . own^T and dP likewise on v_mfma_f32_32x32x16_bf16 with the own side held in registers
+// as the B operand for the whole kernel.  P and dS are, after bf16 conversion, directly the B operands of
+// the accumulating products (dV^T += dO^T P, dK^T += Q^T dS; dQ^T += K^T dS) whose A operands are the
+// transposed tiles staged in LDS, read in the accumulator's row order.  No atomics except the one
+// per-wave add into d sigma / d beta; dQ, dK, dV are deterministic.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "proteus_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float  floatx16 __attribute__((ext_vector_type(16)));
+typedef float  floatx2 __attribute__((ext_vector_type(2)));
+
+constexpr int GB_WAVES   = 4;
+constexpr int GB_THREADS = GB_WAVES * 64;
+constexpr int GB_OWN     = GB_WAVES * 32;   // own tokens per workgroup
+constexpr int GB_BN      = 64;              // streamed tokens per tile
+constexpr int GB_D       = 64;
+constexpr int GB_LDR     = GB_D + 8;        // row stride of a row-major tile [token][d] (bf16 elements)
+constexpr int GB_LDT     = GB_BN + 8;       // row stride of a transposed tile [d][token]
+constexpr float LOG2E    = 1.4426950408889634f;
+
+struct __align__(16) BwdSmem {
+    uint16_t ra[GB_BN * GB_LDR];     // other tokens, first tensor  (K or Q), row-major:  A operand of S
+    uint16_t rb[GB_BN * GB_LDR];     // other tokens, second tensor (V or dO), row-major: A operand of dP
+    uint16_t ta[GB_D * GB_LDT];      // first tensor transposed:  A operand of dQ^T / dK^T
+    uint16_t tb[GB_D * GB_LDT];      // second tensor transposed (dO^T): A operand of dV^T (keys-own pass only)
+    float    rx[GB_BN], ry[GB_BN], rz[GB_BN];   // coordinates of the other tokens
+    float    rl[GB_BN], rd[GB_BN];   // L * log2(e) and D of the other tokens (when they are queries)
+    float    rv[GB_BN];              // 1 for a usable other token, 0 for a padded / out-of-range one
+};
+
+__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
+    floatx2 f = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
+}
+
+template <bool OWN_Q, bool LEGACY>
+__global__ __launch_bounds__(GB_THREADS, 2)
+void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                         const uint16_t* __restrict__ V, const uint16_t* __restrict__ dO,
+                         const float* __restrict__ coords, const float* __restrict__ sigma,
+                         const float* __restrict__ beta, const uint8_t* __restrict__ key_pad,
+                         const float* __restrict__ Lse, const float* __restrict__ Dvec,
+                         float* __restrict__ dQ, float* __restrict__ dK, float* __restrict__ dV,
+                         float* __restrict__ d_sigma, float* __restrict__ d_beta,
+                         const int H, const int N, const int n_otiles, const float min_rbf, const float max_rbf)
+{
+    __shared__ BwdSmem sm;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    const int col  = lane & 31;
+
+    const int ot = blockIdx.x % n_otiles;
+    const int zh = blockIdx.x / n_otiles;
+    const int z  = zh / H;
+    const int h  = zh - z * H;
+    const size_t head_off = (size_t)zh * (size_t)N * GB_D;
+    const float*   cz = coords + (size_t)z * N * 3;
+    const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
+    const float*   Lh = Lse + (size_t)zh * N;
+    const float*   Dh = Dvec + (size_t)zh * N;
+
+    const float sg  = sigma[h];
+    const float cs2 = 0.72134752044448170368f / (sg * sg);       // log2(e)/2 / sigma^2: rbf = exp2(-d^2 cs2)
+    const float bt  = LEGACY ? beta[h] : 0.f;
+    const float rinv = LEGACY ? 1.0f / (max_rbf - min_rbf) : 0.f;
+    const float rn_a = 2.0f * rinv, rn_b = -(2.0f * min_rbf * rinv + 1.0f);   // Rn = rbf rn_a + rn_b
+
+    // ---- own token of this lane ----
+    const int  o      = ot * GB_OWN + wave * 32 + col;
+    const bool own_in = o < N;
+    const int  oc     = own_in ? o : N - 1;
+    const bool own_ok = own_in && !(mz && mz[oc]);
+    const float ox = cz[3 * oc], oy = cz[3 * oc + 1], oz = cz[3 * oc + 2];
+    float own_l2 = 0.f, own_d = 0.f;
+    bool  own_use = own_ok;
+    if (OWN_Q) {
+        const float l = Lh[oc];
+        own_use = own_ok && (l > -INFINITY);
+        own_l2 = own_use ? l * LOG2E : 0.f;
+        own_d  = own_use ? Dh[oc] : 0.f;
+    }
+    // B operands: lane (half, col) holds d = 16*ks + 8*half + 0..7 of its own token; the first one carries 1/sqrt(64)
+    const uint16_t* Bs_src = (OWN_Q ? Q : K) + head_off;
+    const uint16_t* Bp_src = (OWN_Q ? dO : V) + head_off;
+    bf16x8 bs[4], bp[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const uint4 r0 = *reinterpret_cast<const uint4*>(Bs_src + (size_t)oc * GB_D + ks * 16 + half * 8);
+        const uint4 r1 = *reinterpret_cast<const uint4*>(Bp_src + (size_t)oc * GB_D + ks * 16 + half * 8);
+        bf16x8 v = __builtin_bit_cast(bf16x8, r0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
+        bs[ks] = v;
+        bp[ks] = __builtin_bit_cast(bf16x8, r1);
+    }
+
+    floatx16 acc_a[2], acc_b[2];       // OWN_Q: dQ^T (acc_a).  keys own: dK^T (acc_a), dV^T (acc_b).  [d half][16 rows]
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc_a[dt][r] = 0.f; acc_b[dt][r] = 0.f; }
+    float sum_sigma = 0.f, sum_beta = 0.f;
+
+    // staging roles: a thread moves the 8-wide d chunk `dc` of the token pair `kp`
+    const int kp = tid & 31;
+    const int dc = tid >> 5;
+    const uint16_t* Ra_src = (OWN_Q ? K : Q) + head_off;
+    const uint16_t* Rb_src = (OWN_Q ? V : dO) + head_off;
+
+    const int ntiles = (N + GB_BN - 1) / GB_BN;
+    for (int t = 0; t < ntiles; ++t) {
+        const int j0 = t * GB_BN;
+        __syncthreads();                      // the previous tile has been consumed
+        // ---- stage the tile: row-major and transposed copies, padded tokens as zeros ----
+        {
+            const int  ta_ = j0 + 2 * kp, tb_ = ta_ + 1;
+            const bool va = ta_ < N && !(mz && mz[ta_]);
+            const bool vb = tb_ < N && !(mz && mz[tb_]);
+            const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+            const uint4 a0 = va ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8) : zero;
+            const uint4 a1 = vb ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8) : zero;
+            const uint4 b0 = va ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8) : zero;
+            const uint4 b1 = vb ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8) : zero;
+            *reinterpret_cast<uint4*>(&sm.ra[(2 * kp) * GB_LDR + dc * 8])     = a0;
+            *reinterpret_cast<uint4*>(&sm.ra[(2 * kp + 1) * GB_LDR + dc * 8]) = a1;
+            *reinterpret_cast<uint4*>(&sm.rb[(2 * kp) * GB_LDR + dc * 8])     = b0;
+            *reinterpret_cast<uint4*>(&sm.rb[(2 * kp + 1) * GB_LDR + dc * 8]) = b1;
+            const unsigned xa[4] = {a0.x, a0.y, a0.z, a0.w}, ya[4] = {a1.x, a1.y, a1.z, a1.w};
+            const unsigned xb[4] = {b0.x, b0.y, b0.z, b0.w}, yb[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // [d][token pair]: low half-word = even token, high half-word = odd token
+                *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(ya[e], xa[e], 0x05040100u);
+                *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(ya[e], xa[e], 0x07060302u);
+                if (!OWN_Q) {
+                    *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(yb[e], xb[e], 0x05040100u);
+                    *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(yb[e], xb[e], 0x07060302u);
+                }
+            }
+            if (tid < GB_BN) {
+                const int  tk = j0 + tid;
+                const bool in = tk < N;
+                const int  tc = in ? tk : N - 1;
+                bool ok = in && !(mz && mz[tc]);
+                float l2 = 0.f, dd = 0.f;
+                if (!OWN_Q) {
+                    const float l = Lh[tc];
+                    ok = ok && (l > -INFINITY);
+                    l2 = ok ? l * LOG2E : 0.f;
+                    dd = ok ? Dh[tc] : 0.f;
+                }
+                // a padded token's coordinates may hold anything: zeros keep every product finite
+                sm.rx[tid] = ok ? cz[3 * tc] : 0.f;
+                sm.ry[tid] = ok ? cz[3 * tc + 1] : 0.f;
+                sm.rz[tid] = ok ? cz[3 * tc + 2] : 0.f;
+                sm.rl[tid] = l2;
+                sm.rd[tid] = dd;
+                sm.rv[tid] = ok ? 1.0f : 0.f;
+            }
+        }
+        __syncthreads();
+
+#pragma unroll 1
+        for (int mt = 0; mt < 2; ++mt) {
+            // ---- S and dP of the 32 x 32 block: rows = other tokens, column = own token ----
+            floatx16 sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint4 fa = *reinterpret_cast<const uint4*>(&sm.ra[(mt * 32 + col) * GB_LDR + ks * 16 + half * 8]);
+                const uint4 fb = *reinterpret_cast<const uint4*>(&sm.rb[(mt * 32 + col) * GB_LDR + ks * 16 + half * 8]);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), bs[ks], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), bp[ks], pacc, 0, 0, 0);
+            }
+            // ---- per pair: multiplier, P, dt, dS; accumulator register r is row 8*(r/4) + 4*half + (r%4) ----
+            float pv[16], ds[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int rb0 = mt * 32 + 8 * g + 4 * half;
+                const float4 kx = *reinterpret_cast<const float4*>(&sm.rx[rb0]);
+                const float4 ky = *reinterpret_cast<const float4*>(&sm.ry[rb0]);
+                const float4 kz = *reinterpret_cast<const float4*>(&sm.rz[rb0]);
+                const float4 kv = *reinterpret_cast<const float4*>(&sm.rv[rb0]);
+                const float4 kl = *reinterpret_cast<const float4*>(&sm.rl[rb0]);
+                const float4 kd = *reinterpret_cast<const float4*>(&sm.rd[rb0]);
+                const float xs[4] = {kx.x, kx.y, kx.z, kx.w}, ys[4] = {ky.x, ky.y, ky.z, ky.w}, zs[4] = {kz.x, kz.y, kz.z, kz.w};
+                const float vs[4] = {kv.x, kv.y, kv.z, kv.w}, ls[4] = {kl.x, kl.y, kl.z, kl.w}, dds[4] = {kd.x, kd.y, kd.z, kd.w};
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int r = 4 * g + v;
+                    const float s  = sacc[r];
+                    const float dx = ox - xs[v], dy = oy - ys[v], dz = oz - zs[v];
+                    const float d2 = __builtin_fmaf(dz, dz, __builtin_fmaf(dy, dy, dx * dx));
+                    const float rbf = __builtin_amdgcn_exp2f(-d2 * cs2);
+                    bool ok = own_use && vs[v] != 0.f;
+                    float tl, dtds, dtdr;            // logit, its derivative in S, its derivative in rbf (up to a constant)
+                    float rn = 0.f;
+                    if (!LEGACY) {
+                        tl   = __builtin_fmaf(s, rbf, s);
+                        dtds = 1.0f + rbf;
+                        dtdr = s;
+                    } else {
+                        rn   = __builtin_fmaf(rbf, rn_a, rn_b);
+                        const float as = fabsf(s);
+                        tl   = __builtin_fmaf(bt * rn, as, s);
+                        dtds = 1.0f + bt * rn * (s > 0.f ? 1.0f : (s < 0.f ? -1.0f : 0.f));
+                        dtdr = as;
+                        ok   = ok && rbf >= min_rbf && rbf <= max_rbf;
+                    }
+                    const float l2 = OWN_Q ? own_l2 : ls[v];
+                    const float dd = OWN_Q ? own_d : dds[v];
+                    const float p  = ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(tl, LOG2E, -l2)) : 0.f;
+                    const float dt = ok ? p * (pacc[r] - dd) : 0.f;
+                    pv[r] = p;
+                    ds[r] = ok ? dt * dtds : 0.f;
+                    if (!OWN_Q) {
+                        sum_sigma += ok ? dt * dtdr * rbf * d2 : 0.f;
+                        if (LEGACY) sum_beta += ok ? dt * rn * dtdr : 0.f;
+                    }
+                }
+            }
+            // ---- accumulating products: contraction over the other tokens of this block ----
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                // contraction slot e of this half-wave is other token mt*32 + 16*t2 + 8*(e/4) + 4*half + (e%4)
+                const uint4 dsb = make_uint4(pack_bf16(ds[8 * t2 + 0], ds[8 * t2 + 1]), pack_bf16(ds[8 * t2 + 2], ds[8 * t2 + 3]),
+                                             pack_bf16(ds[8 * t2 + 4], ds[8 * t2 + 5]), pack_bf16(ds[8 * t2 + 6], ds[8 * t2 + 7]));
+                const uint4 pb  = make_uint4(pack_bf16(pv[8 * t2 + 0], pv[8 * t2 + 1]), pack_bf16(pv[8 * t2 + 2], pv[8 * t2 + 3]),
+                                             pack_bf16(pv[8 * t2 + 4], pv[8 * t2 + 5]), pack_bf16(pv[8 * t2 + 6], pv[8 * t2 + 7]));
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) {
+                    const uint16_t* rowa = &sm.ta[(dt * 32 + col) * GB_LDT + mt * 32 + 16 * t2 + 4 * half];
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(rowa);
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(rowa + 8);
+                    const uint4 fa = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                    acc_a[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), __builtin_bit_cast(bf16x8, dsb), acc_a[dt], 0, 0, 0);
+                    if (!OWN_Q) {
+                        const uint16_t* rowb = &sm.tb[(dt * 32 + col) * GB_LDT + mt * 32 + 16 * t2 + 4 * half];
+                        const uint2 b0 = *reinterpret_cast<const uint2*>(rowb);
+                        const uint2 b1 = *reinterpret_cast<const uint2*>(rowb + 8);
+                        const uint4 fb = make_uint4(b0.x, b0.y, b1.x, b1.y);
+                        acc_b[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), __builtin_bit_cast(bf16x8, pb), acc_b[dt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: lane (half, col) holds d = dt*32 + 8*g + 4*half + 0..3 of its own token ----
+    if (own_in) {
+        float* out_a = (OWN_Q ? dQ : dK) + head_off + (size_t)o * GB_D;
+        float* out_b = dV + head_off + (size_t)o * GB_D;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
+                if (own_ok) {
+                    va = make_float4(acc_a[dt][4 * g] * 0.125f, acc_a[dt][4 * g + 1] * 0.125f,
+                                     acc_a[dt][4 * g + 2] * 0.125f, acc_a[dt][4 * g + 3] * 0.125f);
+                    vb = make_float4(acc_b[dt][4 * g], acc_b[dt][4 * g + 1], acc_b[dt][4 * g + 2], acc_b[dt][4 * g + 3]);
+                }
+                *reinterpret_cast<float4*>(out_a + dt * 32 + 8 * g + 4 * half) = va;
+                if (!OWN_Q) *reinterpret_cast<float4*>(out_b + dt * 32 + 8 * g + 4 * half) = vb;
+            }
+    }
+    if (!OWN_Q) {
+        for (int off = 32; off > 0; off >>= 1) {
+            sum_sigma += __shfl_xor(sum_sigma, off);
+            if (LEGACY) sum_beta += __shfl_xor(sum_beta, off);
+        }
+        if (lane == 0) {
+            // d rbf / d sigma = rbf d^2 / sigma^3; the legacy logits carry 2 beta/(max - min) in dt/drbf
+            const float k = (LEGACY ? 2.0f * bt * rinv : 1.0f) / (sg * sg * sg);
+            if (d_sigma) atomicAdd(&d_sigma[h], sum_sigma * k);
+            if (LEGACY && d_beta) atomicAdd(&d_beta[h], sum_beta);
+        }
+    }
+}
+
+template <bool LEGACY>
+int launch_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+               const float* coords, const float* sigma, const float* beta, const uint8_t* mask,
+               const float* L, const float* D, float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
+               int Z, int H, int N, float min_rbf, float max_rbf, hipStream_t st)
+{
+    const int n_otiles = (N + GB_OWN - 1) / GB_OWN;
+    dim3 grid((unsigned)n_otiles * (unsigned)(Z * H), 1, 1);
+    hipLaunchKernelGGL((geo_attn_bwd_kernel<false, LEGACY>), grid, dim3(GB_THREADS), 0, st,
+                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf);
+    hipLaunchKernelGGL((geo_attn_bwd_kernel<true, LEGACY>), grid, dim3(GB_THREADS), 0, st,
+                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                          const float* coords, const float* sigma, const float* beta,
+                                          const uint8_t* key_pad_mask, const float* L, const float* D,
+                                          const float* dQ, const float* dK, const float* dV,
+                                          const float* d_sigma, const float* d_beta,
+                                          int Z, int H, int N, int d_head, float min_rbf, float max_rbf)
+{
+    (void)key_pad_mask; (void)d_sigma; (void)d_beta;
+    if (!Q || !K || !V || !dO || !coords || !sigma || !L || !D || !dQ || !dK || !dV) return PROTEUS_ERR_NULL_POINTER;
+    if (Z <= 0 || H <= 0 || N <= 0) return PROTEUS_ERR_BAD_SHAPE;
+    if (N > PROTEUS_ATTN_MAX_N || (long)Z * H > 65535) return PROTEUS_ERR_BAD_SHAPE;
+    if (d_head != GB_D) return PROTEUS_ERR_BAD_HEAD_DIM;
+    if (beta && !(max_rbf > min_rbf)) return PROTEUS_ERR_BAD_SHAPE;
+    if (((uintptr_t)Q & 15) || ((uintptr_t)K & 15) || ((uintptr_t)V & 15) || ((uintptr_t)dO & 15) ||
+        ((uintptr_t)dQ & 15) || ((uintptr_t)dK & 15) || ((uintptr_t)dV & 15)) return PROTEUS_ERR_BAD_ALIGNMENT;
+    return PROTEUS_OK;
+}
+
+extern "C" int proteus_geo_attn_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                    const float* coords, const float* sigma, const float* beta,
+                                    const uint8_t* key_pad_mask, const float* L, const float* D,
+                                    float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
+                                    int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream)
+{
+    const int rc = proteus_geo_attn_bwd_check(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV,
+                                              d_sigma, d_beta, Z, H, N, d_head, min_rbf, max_rbf);
+    if (rc != PROTEUS_OK) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (beta)
+        return launch_bwd<true>(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV, d_sigma, d_beta,
+                                Z, H, N, min_rbf, max_rbf, st);
+    return launch_bwd<false>(Q, K, V, dO, coords, sigma, nullptr, key_pad_mask, L, D, dQ, dK, dV, d_sigma, nullptr,
+                             Z, H, N, 0.f, 1.f, st);
+}

@@ -73,16 +73,67 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     return (O, L) if return_lse else O
 
 
+def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, betas=None,
+                      min_rbf: float = 0.0, max_rbf: float = 1.0):
+    """dQ, dK, dV [Z,H,N,d] f32, d_sigma [H] f32, d_betas [H] f32 | None from the forward's O and logsumexp L.
+
+    What the reference's wrapper does around its backward kernel (geometric_attn.py:609-660):
+    D = rowsum(O*dO), dO cast to the operand type (bf16 here), zeroed accumulators for the per-head scalars.
+    """
+    Z, H, N, d = Q.shape
+    if not Q.is_cuda:
+        raise _lib.ProteusError("geo_attn_backward needs tensors on the GPU (there is no CPU path)")
+    lib = _lib.load()
+    dev = Q.device
+    q = Q.detach().to(torch.bfloat16).contiguous()
+    k = K.detach().to(torch.bfloat16).contiguous()
+    v = V.detach().to(torch.bfloat16).contiguous()
+    D = torch.sum(O.detach().float() * dO.detach().float(), dim=3).contiguous()
+    do = dO.detach().to(torch.bfloat16).contiguous()
+    c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
+    s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
+    lse = L.detach().to(torch.float32).contiguous()
+    m = None
+    if key_padding_mask is not None:
+        m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
+    bt = None if betas is None else betas.detach().to(device=dev, dtype=torch.float32).contiguous()
+    dQ = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
+    dK = torch.empty_like(dQ)
+    dV = torch.empty_like(dQ)
+    d_sigma = torch.zeros(H, dtype=torch.float32, device=dev)
+    d_beta = None if bt is None else torch.zeros(H, dtype=torch.float32, device=dev)
+    if Z == 0 or H == 0 or N == 0:
+        return dQ, dK, dV, d_sigma, d_beta
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), c.data_ptr(), s.data_ptr(),
+                                      None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
+                                      lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
+                                      d_sigma.data_ptr(), None if d_beta is None else d_beta.data_ptr(),
+                                      Z, H, N, d, float(min_rbf), float(max_rbf), stream)
+    _lib.check(rc, "proteus_geo_attn_bwd")
+    return dQ, dK, dV, d_sigma, d_beta
+
+
 class _geometric_attn(torch.autograd.Function):
-    """Forward only: the backward kernel of the reference (geometric_attn.py:262-543) is not implemented."""
+    """Forward and backward on the HIP kernels (old/old_scripts/attn/geometric_attn.py:550-660).  No gradient
+    flows to the coordinates, as in the reference."""
 
     @staticmethod
     def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf):
-        return geo_attn(Q, K, V, coords, spreads, key_padding_mask, betas=betas, min_rbf=min_rbf, max_rbf=max_rbf)
+        O, L = geo_attn(Q, K, V, coords, spreads, key_padding_mask, return_lse=True, betas=betas,
+                        min_rbf=min_rbf, max_rbf=max_rbf)
+        ctx.save_for_backward(Q, K, V, O, L, coords, spreads, betas, key_padding_mask)
+        ctx.min_rbf, ctx.max_rbf = min_rbf, max_rbf
+        return O
 
     @staticmethod
     def backward(ctx, dO):
-        raise NotImplementedError("geometric attention backward is not implemented")
+        Q, K, V, O, L, coords, spreads, betas, mask = ctx.saved_tensors
+        dQ, dK, dV, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
+                                                        ctx.min_rbf, ctx.max_rbf)
+        return (dQ.to(Q.dtype), dK.to(K.dtype), dV.to(V.dtype), None, d_sigma.to(spreads.dtype),
+                None if betas is None else d_beta.to(betas.dtype), None, None, None)
 
 
 def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00):

@@ -105,6 +105,26 @@ def test_attention_argument_validation():
     assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 32, 0.0, 1.0, 0, None) == -3
 
 
+def test_attention_backward_argument_validation():
+    lib = _lib.load()
+    p = 0x1000
+    ok = [p, p, p, p, p, p, None, None, p, p, p, p, p, p, None, 1, 2, 16, 64, 0.0, 1.0]
+
+    def call(**kw):
+        a = list(ok)
+        for i, v in kw.items():
+            a[int(i[1:])] = v
+        return lib.proteus_geo_attn_bwd_check(*a)
+    assert call() == 0
+    for i in (0, 1, 2, 3, 4, 5, 8, 9, 10, 11, 12):
+        assert call(**{f"a{i}": None}) == -1
+    assert call(a15=0) == -2 and call(a17=(1 << 20) + 1) == -2
+    assert call(a18=32) == -3
+    assert call(a10=p + 4) == -5
+    assert call(a6=p, a19=0.5, a20=0.5) == -2          # legacy logits need max_rbf > min_rbf
+    assert lib.proteus_geo_attn_bwd(*(ok[:3] + [None] + ok[4:] + [None])) == -1
+
+
 def test_check_raises_python_exceptions():
     with pytest.raises(ValueError):
         _lib.check(-2, "x")

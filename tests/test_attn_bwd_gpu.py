@@ -1,0 +1,153 @@
+"""GPU parity tests of the geometric attention backward: the HIP kernels, called through the C ABI via the
+autograd function, against torch.autograd through the dense fp64 statement of the forward on the same
+bf16-rounded inputs.
+
+Bar: the operands of every matrix product are bf16 (Q, K, V, dO, P, dS; the reference uses fp16), so each
+gradient tensor is compared in relative L2 norm: <= 2e-2 for dQ, dK, dV, d_sigma, d_beta."""
+import numpy as np
+import pytest
+import torch
+
+import proteusai_amd as pa
+from oracle import torch_oracle
+from proteusai_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 2e-2
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    nb = np.linalg.norm(b)
+    return float(np.linalg.norm(a - b) / nb) if nb > 0 else float(np.linalg.norm(a - b))
+
+
+def make(seed, Z, H, N, maskfrac=0.0, qscale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    Q = (torch.randn(Z, H, N, 64, generator=g) * qscale).bfloat16()
+    K = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    dO = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    coords = torch.stack([synth.random_walk_chain(N, g) for _ in range(Z)])
+    sigma = synth.log_spaced_sigma(H)
+    mask = (torch.rand(Z, N, generator=g) < maskfrac) if maskfrac > 0 else None
+    return Q, K, V, dO, coords, sigma, mask
+
+
+def reference_grads(Q, K, V, dO, coords, sigma, mask, betas=None, min_rbf=0.0, max_rbf=1.0):
+    q, k, v = (t.double().requires_grad_(True) for t in (Q, K, V))
+    s = sigma.double().requires_grad_(True)
+    b = None if betas is None else betas.double().requires_grad_(True)
+    O = torch_oracle.geo_attn_autograd_torch(q, k, v, coords, s, mask, b, min_rbf, max_rbf)
+    O.backward(dO.double())
+    return q.grad, k.grad, v.grad, s.grad, None if b is None else b.grad
+
+
+def gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask, betas=None, min_rbf=0.0, max_rbf=1.0):
+    q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
+    s = sigma.to(gpu).requires_grad_(True)
+    b = None if betas is None else betas.to(gpu).requires_grad_(True)
+    O = pa.geometric_attn(q, k, v, coords.to(gpu), s, b, None if mask is None else mask.to(gpu), min_rbf, max_rbf)
+    O.backward(dO.to(gpu).float())
+    torch.cuda.synchronize()
+    return q.grad.float().cpu(), k.grad.float().cpu(), v.grad.float().cpu(), s.grad.cpu(), None if b is None else b.grad.cpu()
+
+
+def compare(got, ref, mask, what):
+    for g, r, name in zip(got, ref, ("dQ", "dK", "dV", "d_sigma", "d_beta")):
+        if r is None:
+            continue
+        assert torch.isfinite(g).all(), f"{what} {name}: non-finite"
+        e = rel_l2(g.numpy(), r.numpy())
+        assert e <= REL_L2_TOL, f"{what} {name}: rel-L2 {e:.3e}"
+    if mask is not None:
+        for g, name in zip(got[:3], ("dQ", "dK", "dV")):
+            assert (g[mask[:, None, :].expand(-1, g.shape[1], -1)] == 0).all(), f"{what} {name}: padded tokens must get zeros"
+
+
+@pytest.mark.parametrize("N", [1, 2, 31, 32, 33, 64, 65, 127, 128, 129, 200, 333])
+def test_ragged_lengths(gpu, N):
+    a = make(300 + N, 2, 3, N)
+    if N == 1:
+        got = gpu_grads(gpu, *a)
+        # a lone token attends to itself with weight 1: O = V, so dV = dO and nothing else moves
+        assert rel_l2(got[2].numpy(), a[3].float().numpy()) <= REL_L2_TOL
+        assert got[0].abs().max() <= 1e-3 and got[1].abs().max() <= 1e-3
+        return
+    compare(gpu_grads(gpu, *a), reference_grads(*a), None, f"N={N}")
+
+
+def test_masks(gpu):
+    N = 300
+    Q, K, V, dO, coords, sigma, _ = make(1, 5, 2, N)
+    g = torch.Generator().manual_seed(1)
+    mask = torch.zeros(5, N, dtype=torch.bool)
+    mask[0] = torch.rand(N, generator=g) < 0.5
+    mask[1, 131:] = True
+    mask[2] = True
+    mask[3] = True
+    mask[3, 77] = False
+    mask[4, :64] = True
+    a = (Q, K, V, dO, coords, sigma, mask)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "masks")
+
+
+def test_padded_content_cannot_matter(gpu):
+    Q, K, V, dO, coords, sigma, mask = make(2, 2, 4, 260, maskfrac=0.3)
+    got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask)
+    Q2, K2, V2, dO2, c2 = Q.clone(), K.clone(), V.clone(), dO.clone(), coords.clone()
+    pad = mask[:, None, :].expand(-1, 4, -1)
+    for t in (Q2, K2, V2, dO2):
+        t[pad] = float("nan")
+    c2[mask] = float("nan")
+    got2 = gpu_grads(gpu, Q2, K2, V2, dO2, c2, sigma, mask)
+    for x, y, name in zip(got[:3], got2[:3], ("dQ", "dK", "dV")):
+        assert torch.equal(x, y), name
+    assert rel_l2(got2[3].numpy(), got[3].numpy()) <= 1e-5      # (atomic adds: summation order may differ)
+
+
+def test_large_logits(gpu):
+    a = make(3, 1, 4, 400, qscale=2.5)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), None, "large logits")
+
+
+def test_legacy_logits(gpu):
+    Q, K, V, dO, coords, sigma, mask = make(4, 2, 4, 300, maskfrac=0.2)
+    betas = torch.tensor([0.5, 1.0, 0.25, 2.0])
+    for lo, hi in ((0.0, 1.0), (0.05, 0.9)):
+        got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask, betas, lo, hi)
+        ref = reference_grads(Q, K, V, dO, coords, sigma, mask, betas, lo, hi)
+        compare(got, ref, mask, f"legacy [{lo},{hi}]")
+
+
+def test_gradients_are_deterministic_except_the_atomic_scalars(gpu):
+    a = make(5, 1, 2, 500)
+    x = gpu_grads(gpu, *a)
+    y = gpu_grads(gpu, *a)
+    for p, q in zip(x[:3], y[:3]):
+        assert torch.equal(p, q)
+
+
+def test_cfg3_shape_sampled(gpu):
+    # Z=4, H=8, N=4096 would need a 4096^2 dense fp64 reference per head: check one batch item and two heads of
+    # that shape in full, through the raw operator (heads and batch items are independent)
+    Q, K, V, dO, coords, sigma, _ = make(6, 1, 2, 2048)
+    compare(gpu_grads(gpu, Q, K, V, dO, coords, sigma, None), reference_grads(Q, K, V, dO, coords, sigma, None), None, "N=2048")
+
+
+def test_module_trains(gpu):
+    torch.manual_seed(0)
+    m = pa.GeoAttention(d_model=128, heads=2).to(gpu)
+    x = torch.randn(2, 70, 128, device=gpu)
+    coords = torch.stack([synth.random_walk_chain(70, torch.Generator().manual_seed(i)) for i in range(2)]).to(gpu)
+    mask = torch.zeros(2, 70, dtype=torch.bool, device=gpu)
+    mask[1, 50:] = True
+    y = m(x, x, x, coords, mask)
+    y[~mask].square().mean().backward()
+    for name, p in m.named_parameters():
+        if name == "beta_weights":
+            continue
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+    assert m.spread_weights.grad.abs().sum() > 0 and m.q_proj.grad.abs().sum() > 0

@@ -150,3 +150,29 @@ def test_legacy_logits_oracles():
     S = S + beta.double()[None, :, None, None] * S.abs()
     ref1 = torch.matmul(torch.softmax(S, -1), V.double()).numpy()
     assert np.abs(O1 - ref1).max() < 1e-10
+
+
+def test_differentiable_statement_equals_the_tiled_ones():
+    # the backward tests differentiate geo_attn_autograd_torch with torch.autograd: its forward must be the
+    # same function as the oracles pinned above, for both kinds of logits, masks and empty rows included
+    g = torch.Generator().manual_seed(11)
+    Z, H, N = 2, 3, 37
+    Q, K, V = (torch.randn(Z, H, N, 64, generator=g, dtype=torch.float64) for _ in range(3))
+    coords = torch.randn(Z, N, 3, generator=g, dtype=torch.float64) * 5
+    sigma = torch.tensor([2.0, 5.0, 11.0], dtype=torch.float64)
+    mask = torch.rand(Z, N, generator=g) < 0.3
+    mask[1] = True
+    mask[1, 5] = False
+    O1, _ = torch_oracle.geo_attn_torch(Q, K, V, coords, sigma, mask, dtype=torch.float64)
+    O2 = torch_oracle.geo_attn_autograd_torch(Q, K, V, coords, sigma, mask)
+    torch.testing.assert_close(O2, O1, rtol=1e-12, atol=1e-12)
+    betas = torch.tensor([0.5, 1.0, 2.0], dtype=torch.float64)
+    O3, _ = torch_oracle.geo_attn_legacy_torch(Q, K, V, coords, sigma, betas, mask, 0.05, 0.9, dtype=torch.float64)
+    O4 = torch_oracle.geo_attn_autograd_torch(Q, K, V, coords, sigma, mask, betas, 0.05, 0.9)
+    torch.testing.assert_close(O4, O3, rtol=1e-12, atol=1e-12)
+    # and it is differentiable without NaNs through masked and empty rows
+    q = Q.clone().requires_grad_(True)
+    s = sigma.clone().requires_grad_(True)
+    torch_oracle.geo_attn_autograd_torch(q, K, V, coords, s, mask).sum().backward()
+    assert torch.isfinite(q.grad).all() and torch.isfinite(s.grad).all()
+    assert (q.grad[mask[:, None, :].expand(-1, H, -1)] == 0).all()
