@@ -134,57 +134,67 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const uint16_t* Ra_src = (OWN_Q ? K : Q) + head_off;
     const uint16_t* Rb_src = (OWN_Q ? V : dO) + head_off;
 
-    const int ntiles = (N + GB_BN - 1) / GB_BN;
-    for (int t = 0; t < ntiles; ++t) {
-        const int j0 = t * GB_BN;
-        __syncthreads();                      // the previous tile has been consumed
-        // ---- stage the tile: row-major and transposed copies, padded tokens as zeros ----
-        {
-            const int  ta_ = j0 + 2 * kp, tb_ = ta_ + 1;
-            const bool va = ta_ < N && !(mz && mz[ta_]);
-            const bool vb = tb_ < N && !(mz && mz[tb_]);
-            const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-            const uint4 a0 = va ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8) : zero;
-            const uint4 a1 = vb ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8) : zero;
-            const uint4 b0 = va ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8) : zero;
-            const uint4 b1 = vb ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8) : zero;
-            *reinterpret_cast<uint4*>(&sm.ra[(2 * kp) * GB_LDR + dc * 8])     = a0;
-            *reinterpret_cast<uint4*>(&sm.ra[(2 * kp + 1) * GB_LDR + dc * 8]) = a1;
-            *reinterpret_cast<uint4*>(&sm.rb[(2 * kp) * GB_LDR + dc * 8])     = b0;
-            *reinterpret_cast<uint4*>(&sm.rb[(2 * kp + 1) * GB_LDR + dc * 8]) = b1;
-            const unsigned xa[4] = {a0.x, a0.y, a0.z, a0.w}, ya[4] = {a1.x, a1.y, a1.z, a1.w};
-            const unsigned xb[4] = {b0.x, b0.y, b0.z, b0.w}, yb[4] = {b1.x, b1.y, b1.z, b1.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // [d][token pair]: low half-word = even token, high half-word = odd token
-                *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(ya[e], xa[e], 0x05040100u);
-                *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(ya[e], xa[e], 0x07060302u);
-                if (!OWN_Q) {
-                    *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(yb[e], xb[e], 0x05040100u);
-                    *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(yb[e], xb[e], 0x07060302u);
-                }
+    // registers holding the tile in flight from global memory: requested before the current tile is
+    // computed, written to LDS after it (padded tokens as zeros)
+    uint4 ga0, ga1, gb0, gb1;
+    float gx = 0.f, gy = 0.f, gz = 0.f, gl = 0.f, gd = 0.f, gv = 0.f;
+    auto load_tile = [&](const int j0) {
+        const int  ta_ = j0 + 2 * kp, tb_ = ta_ + 1;
+        const bool va = ta_ < N && !(mz && mz[ta_]);
+        const bool vb = tb_ < N && !(mz && mz[tb_]);
+        const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+        ga0 = va ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8) : zero;
+        ga1 = vb ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8) : zero;
+        gb0 = va ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8) : zero;
+        gb1 = vb ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8) : zero;
+        if (tid < GB_BN) {
+            const int  tk = j0 + tid;
+            const bool in = tk < N;
+            const int  tc = in ? tk : N - 1;
+            bool ok = in && !(mz && mz[tc]);
+            float l2 = 0.f, dd = 0.f;
+            if (!OWN_Q) {
+                const float l = Lh[tc];
+                ok = ok && (l > -INFINITY);
+                l2 = ok ? l * LOG2E : 0.f;
+                dd = ok ? Dh[tc] : 0.f;
             }
-            if (tid < GB_BN) {
-                const int  tk = j0 + tid;
-                const bool in = tk < N;
-                const int  tc = in ? tk : N - 1;
-                bool ok = in && !(mz && mz[tc]);
-                float l2 = 0.f, dd = 0.f;
-                if (!OWN_Q) {
-                    const float l = Lh[tc];
-                    ok = ok && (l > -INFINITY);
-                    l2 = ok ? l * LOG2E : 0.f;
-                    dd = ok ? Dh[tc] : 0.f;
-                }
-                // a padded token's coordinates may hold anything: zeros keep every product finite
-                sm.rx[tid] = ok ? cz[3 * tc] : 0.f;
-                sm.ry[tid] = ok ? cz[3 * tc + 1] : 0.f;
-                sm.rz[tid] = ok ? cz[3 * tc + 2] : 0.f;
-                sm.rl[tid] = l2;
-                sm.rd[tid] = dd;
-                sm.rv[tid] = ok ? 1.0f : 0.f;
+            // a padded token's coordinates may hold anything: zeros keep every product finite
+            gx = ok ? cz[3 * tc] : 0.f;
+            gy = ok ? cz[3 * tc + 1] : 0.f;
+            gz = ok ? cz[3 * tc + 2] : 0.f;
+            gl = l2; gd = dd; gv = ok ? 1.0f : 0.f;
+        }
+    };
+    auto store_tile = [&]() {
+        *reinterpret_cast<uint4*>(&sm.ra[(2 * kp) * GB_LDR + dc * 8])     = ga0;
+        *reinterpret_cast<uint4*>(&sm.ra[(2 * kp + 1) * GB_LDR + dc * 8]) = ga1;
+        *reinterpret_cast<uint4*>(&sm.rb[(2 * kp) * GB_LDR + dc * 8])     = gb0;
+        *reinterpret_cast<uint4*>(&sm.rb[(2 * kp + 1) * GB_LDR + dc * 8]) = gb1;
+        const unsigned xa[4] = {ga0.x, ga0.y, ga0.z, ga0.w}, ya[4] = {ga1.x, ga1.y, ga1.z, ga1.w};
+        const unsigned xb[4] = {gb0.x, gb0.y, gb0.z, gb0.w}, yb[4] = {gb1.x, gb1.y, gb1.z, gb1.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            // [d][token pair]: low half-word = even token, high half-word = odd token
+            *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(ya[e], xa[e], 0x05040100u);
+            *reinterpret_cast<unsigned*>(&sm.ta[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(ya[e], xa[e], 0x07060302u);
+            if (!OWN_Q) {
+                *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e) * GB_LDT + 2 * kp])     = __builtin_amdgcn_perm(yb[e], xb[e], 0x05040100u);
+                *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(yb[e], xb[e], 0x07060302u);
             }
         }
+        if (tid < GB_BN) {
+            sm.rx[tid] = gx; sm.ry[tid] = gy; sm.rz[tid] = gz;
+            sm.rl[tid] = gl; sm.rd[tid] = gd; sm.rv[tid] = gv;
+        }
+    };
+
+    const int ntiles = (N + GB_BN - 1) / GB_BN;
+    load_tile(0);
+    for (int t = 0; t < ntiles; ++t) {
+        __syncthreads();                      // the previous tile has been consumed
+        store_tile();
+        if (t + 1 < ntiles) load_tile((t + 1) * GB_BN);
         __syncthreads();
 
 #pragma unroll 1
