@@ -24,6 +24,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "proteus_hip.h"
 
 namespace {
@@ -48,8 +49,9 @@ struct __align__(16) BwdSmem {
     uint16_t ta[GB_D * GB_LDT];      // first tensor transposed:  A operand of dQ^T / dK^T
     uint16_t tb[GB_D * GB_LDT];      // second tensor transposed (dO^T): A operand of dV^T (keys-own pass only)
     float    rx[GB_BN], ry[GB_BN], rz[GB_BN];   // coordinates of the other tokens
-    float    rl[GB_BN], rd[GB_BN];   // L * log2(e) and D of the other tokens (when they are queries)
-    float    rv[GB_BN];              // 1 for a usable other token, 0 for a padded / out-of-range one
+    float    rl[GB_BN], rd[GB_BN];   // per other token: L*log2(e) if it is a usable query, 0 if a usable key, +inf if
+                                     // unusable (padded / out of range / empty row); D of a usable query, else 0
+    float    box[8];                 // bounding box of the usable other tokens of the tile: lo xyz, hi xyz
 };
 
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
@@ -97,15 +99,27 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const bool own_in = o < N;
     const int  oc     = own_in ? o : N - 1;
     const bool own_ok = own_in && !(mz && mz[oc]);
-    const float ox = cz[3 * oc], oy = cz[3 * oc + 1], oz = cz[3 * oc + 2];
-    float own_l2 = 0.f, own_d = 0.f;
+    // An unusable own token (padded, out of range, or a query without any unmasked pair) is given zero
+    // operands, zero coordinates and an exponent offset of +inf: every pair with it gets P = exp2(-inf) = 0
+    // and all its products stay finite, without a select per pair.
     bool  own_use = own_ok;
+    float own_l2 = 0.f, own_d = 0.f;
     if (OWN_Q) {
         const float l = Lh[oc];
         own_use = own_ok && (l > -INFINITY);
         own_l2 = own_use ? l * LOG2E : 0.f;
         own_d  = own_use ? Dh[oc] : 0.f;
     }
+    if (!own_use) own_l2 = INFINITY;
+    const float ox = own_use ? cz[3 * oc] : 0.f, oy = own_use ? cz[3 * oc + 1] : 0.f, oz = own_use ? cz[3 * oc + 2] : 0.f;
+    // bounding box of the wave's usable own tokens (for the far-tile test)
+    float blo[3] = {own_use ? ox : 3.0e38f, own_use ? oy : 3.0e38f, own_use ? oz : 3.0e38f};
+    float bhi[3] = {own_use ? ox : -3.0e38f, own_use ? oy : -3.0e38f, own_use ? oz : -3.0e38f};
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+        for (int off = 32; off > 0; off >>= 1) { blo[c] = fminf(blo[c], __shfl_xor(blo[c], off)); bhi[c] = fmaxf(bhi[c], __shfl_xor(bhi[c], off)); }
+    // exp2(-d^2 cs2) < 2^-25 beyond this distance: s*(1+rbf) rounds to s in fp32
+    const float far2 = 25.0f / cs2;
     // B operands: lane (half, col) holds d = 16*ks + 8*half + 0..7 of its own token; the first one carries 1/sqrt(64)
     const uint16_t* Bs_src = (OWN_Q ? Q : K) + head_off;
     const uint16_t* Bp_src = (OWN_Q ? dO : V) + head_off;
@@ -114,11 +128,11 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     for (int ks = 0; ks < 4; ++ks) {
         const uint4 r0 = *reinterpret_cast<const uint4*>(Bs_src + (size_t)oc * GB_D + ks * 16 + half * 8);
         const uint4 r1 = *reinterpret_cast<const uint4*>(Bp_src + (size_t)oc * GB_D + ks * 16 + half * 8);
-        bf16x8 v = __builtin_bit_cast(bf16x8, r0);
+        bf16x8 v = __builtin_bit_cast(bf16x8, own_use ? r0 : make_uint4(0u, 0u, 0u, 0u));
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
         bs[ks] = v;
-        bp[ks] = __builtin_bit_cast(bf16x8, r1);
+        bp[ks] = __builtin_bit_cast(bf16x8, own_use ? r1 : make_uint4(0u, 0u, 0u, 0u));
     }
 
     floatx16 acc_a[2], acc_b[2];       // OWN_Q: dQ^T (acc_a).  keys own: dK^T (acc_a), dV^T (acc_b).  [d half][16 rows]
@@ -127,6 +141,10 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
         for (int r = 0; r < 16; ++r) { acc_a[dt][r] = 0.f; acc_b[dt][r] = 0.f; }
     float sum_sigma = 0.f, sum_beta = 0.f;
+    // log2(e) in a vector register: as a literal it would make each instruction that uses it a
+    // scalar-operand one (4 clocks instead of about 2.5)
+    float log2e_v = LOG2E;
+    asm volatile("" : "+v"(log2e_v));
 
     // staging roles: a thread moves the 8-wide d chunk `dc` of the token pair `kp`
     const int kp = tid & 31;
@@ -137,7 +155,8 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // registers holding the tile in flight from global memory: requested before the current tile is
     // computed, written to LDS after it (padded tokens as zeros)
     uint4 ga0, ga1, gb0, gb1;
-    float gx = 0.f, gy = 0.f, gz = 0.f, gl = 0.f, gd = 0.f, gv = 0.f;
+    float gx = 0.f, gy = 0.f, gz = 0.f, gl = 0.f, gd = 0.f;
+    bool  gok = false;
     auto load_tile = [&](const int j0) {
         const int  ta_ = j0 + 2 * kp, tb_ = ta_ + 1;
         const bool va = ta_ < N && !(mz && mz[ta_]);
@@ -163,7 +182,7 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             gx = ok ? cz[3 * tc] : 0.f;
             gy = ok ? cz[3 * tc + 1] : 0.f;
             gz = ok ? cz[3 * tc + 2] : 0.f;
-            gl = l2; gd = dd; gv = ok ? 1.0f : 0.f;
+            gl = ok ? l2 : INFINITY; gd = dd; gok = ok;
         }
     };
     auto store_tile = [&]() {
@@ -183,9 +202,18 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 *reinterpret_cast<unsigned*>(&sm.tb[(dc * 8 + 2 * e + 1) * GB_LDT + 2 * kp]) = __builtin_amdgcn_perm(yb[e], xb[e], 0x07060302u);
             }
         }
-        if (tid < GB_BN) {
+        if (tid < GB_BN) {       // = wave 0, one token per lane
             sm.rx[tid] = gx; sm.ry[tid] = gy; sm.rz[tid] = gz;
-            sm.rl[tid] = gl; sm.rd[tid] = gd; sm.rv[tid] = gv;
+            sm.rl[tid] = gl; sm.rd[tid] = gd;
+            float lo[3] = {gok ? gx : 3.0e38f, gok ? gy : 3.0e38f, gok ? gz : 3.0e38f};
+            float hi[3] = {gok ? gx : -3.0e38f, gok ? gy : -3.0e38f, gok ? gz : -3.0e38f};
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                for (int off = 32; off > 0; off >>= 1) { lo[c] = fminf(lo[c], __shfl_xor(lo[c], off)); hi[c] = fmaxf(hi[c], __shfl_xor(hi[c], off)); }
+            if (tid == 0) {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) { sm.box[c] = lo[c]; sm.box[3 + c] = hi[c]; }
+            }
         }
     };
 
@@ -196,6 +224,20 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         store_tile();
         if (t + 1 < ntiles) load_tile((t + 1) * GB_BN);
         __syncthreads();
+
+        // far-tile test: distance between the box of this wave's own tokens and the box of the tile's tokens.
+        // Beyond `far2` the multiplier is 1 to fp32 rounding and its derivative terms vanish, so the geometry
+        // is skipped for the whole tile (the legacy logits depend on rbf down to 0: always evaluated).
+        bool near = true;
+        if (!LEGACY) {
+            float g2 = 0.f;
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                const float gap = fmaxf(fmaxf(blo[c] - sm.box[3 + c], sm.box[c] - bhi[c]), 0.f);
+                g2 = __builtin_fmaf(gap, gap, g2);
+            }
+            near = !(g2 > far2);             // (an empty box gives an infinite gap: far, and every P is 0 anyway)
+        }
 
 #pragma unroll 1
         for (int mt = 0; mt < 2; ++mt) {
@@ -210,53 +252,72 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), bs[ks], sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), bp[ks], pacc, 0, 0, 0);
             }
-            // ---- per pair: multiplier, P, dt, dS; accumulator register r is row 8*(r/4) + 4*half + (r%4) ----
+            // ---- per pair: multiplier, P, dt, dS; accumulator register r is row 8*(r/4) + 4*half + (r%4).
+            // Unusable tokens carry +inf in their exponent offset: P = exp2(-inf) = 0, and since their
+            // operands and coordinates are zeros everything derived from P is an exact 0 as well. ----
             float pv[16], ds[16];
+            auto pairs = [&](auto near_c) {
+                constexpr bool NEAR = decltype(near_c)::value;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int rb0 = mt * 32 + 8 * g + 4 * half;
-                const float4 kx = *reinterpret_cast<const float4*>(&sm.rx[rb0]);
-                const float4 ky = *reinterpret_cast<const float4*>(&sm.ry[rb0]);
-                const float4 kz = *reinterpret_cast<const float4*>(&sm.rz[rb0]);
-                const float4 kv = *reinterpret_cast<const float4*>(&sm.rv[rb0]);
-                const float4 kl = *reinterpret_cast<const float4*>(&sm.rl[rb0]);
-                const float4 kd = *reinterpret_cast<const float4*>(&sm.rd[rb0]);
-                const float xs[4] = {kx.x, kx.y, kx.z, kx.w}, ys[4] = {ky.x, ky.y, ky.z, ky.w}, zs[4] = {kz.x, kz.y, kz.z, kz.w};
-                const float vs[4] = {kv.x, kv.y, kv.z, kv.w}, ls[4] = {kl.x, kl.y, kl.z, kl.w}, dds[4] = {kd.x, kd.y, kd.z, kd.w};
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int r = 4 * g + v;
-                    const float s  = sacc[r];
-                    const float dx = ox - xs[v], dy = oy - ys[v], dz = oz - zs[v];
-                    const float d2 = __builtin_fmaf(dz, dz, __builtin_fmaf(dy, dy, dx * dx));
-                    const float rbf = __builtin_amdgcn_exp2f(-d2 * cs2);
-                    bool ok = own_use && vs[v] != 0.f;
-                    float tl, dtds, dtdr;            // logit, its derivative in S, its derivative in rbf (up to a constant)
-                    float rn = 0.f;
-                    if (!LEGACY) {
-                        tl   = __builtin_fmaf(s, rbf, s);
-                        dtds = 1.0f + rbf;
-                        dtdr = s;
-                    } else {
-                        rn   = __builtin_fmaf(rbf, rn_a, rn_b);
-                        const float as = fabsf(s);
-                        tl   = __builtin_fmaf(bt * rn, as, s);
-                        dtds = 1.0f + bt * rn * (s > 0.f ? 1.0f : (s < 0.f ? -1.0f : 0.f));
-                        dtdr = as;
-                        ok   = ok && rbf >= min_rbf && rbf <= max_rbf;
+                for (int g = 0; g < 4; ++g) {
+                    const int rb0 = mt * 32 + 8 * g + 4 * half;
+                    const float4 kl = *reinterpret_cast<const float4*>(&sm.rl[rb0]);
+                    const float ls[4] = {kl.x, kl.y, kl.z, kl.w};
+                    float xs[4] = {0.f, 0.f, 0.f, 0.f}, ys[4] = {0.f, 0.f, 0.f, 0.f}, zs[4] = {0.f, 0.f, 0.f, 0.f};
+                    float dds[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (NEAR) {
+                        const float4 kx = *reinterpret_cast<const float4*>(&sm.rx[rb0]);
+                        const float4 ky = *reinterpret_cast<const float4*>(&sm.ry[rb0]);
+                        const float4 kz = *reinterpret_cast<const float4*>(&sm.rz[rb0]);
+                        xs[0] = kx.x; xs[1] = kx.y; xs[2] = kx.z; xs[3] = kx.w;
+                        ys[0] = ky.x; ys[1] = ky.y; ys[2] = ky.z; ys[3] = ky.w;
+                        zs[0] = kz.x; zs[1] = kz.y; zs[2] = kz.z; zs[3] = kz.w;
                     }
-                    const float l2 = OWN_Q ? own_l2 : ls[v];
-                    const float dd = OWN_Q ? own_d : dds[v];
-                    const float p  = ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(tl, LOG2E, -l2)) : 0.f;
-                    const float dt = ok ? p * (pacc[r] - dd) : 0.f;
-                    pv[r] = p;
-                    ds[r] = ok ? dt * dtds : 0.f;
                     if (!OWN_Q) {
-                        sum_sigma += ok ? dt * dtdr * rbf * d2 : 0.f;
-                        if (LEGACY) sum_beta += ok ? dt * rn * dtdr : 0.f;
+                        const float4 kd = *reinterpret_cast<const float4*>(&sm.rd[rb0]);
+                        dds[0] = kd.x; dds[1] = kd.y; dds[2] = kd.z; dds[3] = kd.w;
+                    }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int r = 4 * g + v;
+                        const float s  = sacc[r];
+                        const float off = -(ls[v] + own_l2);          // -(L log2e) of the pair's query, -inf if unusable
+                        const float dd = OWN_Q ? own_d : dds[v];
+                        if (!NEAR) {
+                            const float p  = __builtin_amdgcn_exp2f(__builtin_fmaf(s, log2e_v, off));
+                            const float dt = p * (pacc[r] - dd);
+                            pv[r] = p;
+                            ds[r] = dt;
+                            continue;
+                        }
+                        const float dx = ox - xs[v], dy = oy - ys[v], dz = oz - zs[v];
+                        const float d2 = __builtin_fmaf(dz, dz, __builtin_fmaf(dy, dy, dx * dx));
+                        const float rbf = __builtin_amdgcn_exp2f(-d2 * cs2);
+                        if (!LEGACY) {
+                            const float tl = __builtin_fmaf(s, rbf, s);
+                            const float p  = __builtin_amdgcn_exp2f(__builtin_fmaf(tl, log2e_v, off));
+                            const float dt = p * (pacc[r] - dd);
+                            pv[r] = p;
+                            ds[r] = __builtin_fmaf(dt, rbf, dt);                    // dt/dS = 1 + rbf
+                            if (!OWN_Q) sum_sigma = __builtin_fmaf(dt * s, rbf * d2, sum_sigma);   // dt/drbf = S
+                        } else {
+                            const float rn = __builtin_fmaf(rbf, rn_a, rn_b);
+                            const float as = fabsf(s);
+                            const float tl = __builtin_fmaf(bt * rn, as, s);
+                            const bool  in_range = rbf >= min_rbf && rbf <= max_rbf;
+                            const float p  = in_range ? __builtin_amdgcn_exp2f(__builtin_fmaf(tl, log2e_v, off)) : 0.f;
+                            const float dt = p * (pacc[r] - dd);
+                            pv[r] = p;
+                            ds[r] = dt * (1.0f + bt * rn * (s > 0.f ? 1.0f : (s < 0.f ? -1.0f : 0.f)));
+                            if (!OWN_Q) {
+                                sum_sigma = __builtin_fmaf(dt * as, rbf * d2, sum_sigma);
+                                sum_beta  = __builtin_fmaf(dt * rn, as, sum_beta);
+                            }
+                        }
                     }
                 }
-            }
+            };
+            if (near) pairs(std::true_type{}); else pairs(std::false_type{});
             // ---- accumulating products: contraction over the other tokens of this block ----
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
