@@ -156,36 +156,32 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // computed, written to LDS after it (padded tokens as zeros)
     uint4 ga0, ga1, gb0, gb1;
     float gx = 0.f, gy = 0.f, gz = 0.f, gl = 0.f, gd = 0.f;
-    bool  gok = false;
+    unsigned gm0 = 0, gm1 = 0, gm = 0;      // raw padding bytes of the two staged tokens / of token tid
+    int gj0 = 0;
+    // Only requests: every address is clamped into range and nothing that comes back is looked at before
+    // store_tile, so no load waits for another.
     auto load_tile = [&](const int j0) {
-        const int  ta_ = j0 + 2 * kp, tb_ = ta_ + 1;
-        const bool va = ta_ < N && !(mz && mz[ta_]);
-        const bool vb = tb_ < N && !(mz && mz[tb_]);
-        const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-        ga0 = va ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8) : zero;
-        ga1 = vb ? *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8) : zero;
-        gb0 = va ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8) : zero;
-        gb1 = vb ? *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8) : zero;
+        gj0 = j0;
+        const int ta_ = min(j0 + 2 * kp, N - 1), tb_ = min(j0 + 2 * kp + 1, N - 1);
+        ga0 = *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8);
+        ga1 = *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8);
+        gb0 = *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8);
+        gb1 = *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8);
+        if (mz) { gm0 = mz[ta_]; gm1 = mz[tb_]; }
         if (tid < GB_BN) {
-            const int  tk = j0 + tid;
-            const bool in = tk < N;
-            const int  tc = in ? tk : N - 1;
-            bool ok = in && !(mz && mz[tc]);
-            float l2 = 0.f, dd = 0.f;
-            if (!OWN_Q) {
-                const float l = Lh[tc];
-                ok = ok && (l > -INFINITY);
-                l2 = ok ? l * LOG2E : 0.f;
-                dd = ok ? Dh[tc] : 0.f;
-            }
-            // a padded token's coordinates may hold anything: zeros keep every product finite
-            gx = ok ? cz[3 * tc] : 0.f;
-            gy = ok ? cz[3 * tc + 1] : 0.f;
-            gz = ok ? cz[3 * tc + 2] : 0.f;
-            gl = ok ? l2 : INFINITY; gd = dd; gok = ok;
+            const int tc = min(j0 + tid, N - 1);
+            gx = cz[3 * tc]; gy = cz[3 * tc + 1]; gz = cz[3 * tc + 2];
+            if (mz) gm = mz[tc];
+            if (!OWN_Q) { gl = Lh[tc]; gd = Dh[tc]; }
         }
     };
     auto store_tile = [&]() {
+        {
+            // padded / out-of-range tokens as zeros
+            const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+            if (gj0 + 2 * kp >= N || gm0) { ga0 = zero; gb0 = zero; }
+            if (gj0 + 2 * kp + 1 >= N || gm1) { ga1 = zero; gb1 = zero; }
+        }
         *reinterpret_cast<uint4*>(&sm.ra[(2 * kp) * GB_LDR + dc * 8])     = ga0;
         *reinterpret_cast<uint4*>(&sm.ra[(2 * kp + 1) * GB_LDR + dc * 8]) = ga1;
         *reinterpret_cast<uint4*>(&sm.rb[(2 * kp) * GB_LDR + dc * 8])     = gb0;
@@ -203,6 +199,11 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             }
         }
         if (tid < GB_BN) {       // = wave 0, one token per lane
+            bool gok = (gj0 + tid < N) && gm == 0;
+            if (!OWN_Q) gok = gok && (gl > -INFINITY);
+            // an unusable token's coordinates, L and D may hold anything: zeros keep every product finite
+            if (!gok) { gx = 0.f; gy = 0.f; gz = 0.f; gd = 0.f; }
+            gl = gok ? (OWN_Q ? 0.f : gl * LOG2E) : INFINITY;
             sm.rx[tid] = gx; sm.ry[tid] = gy; sm.rz[tid] = gz;
             sm.rl[tid] = gl; sm.rd[tid] = gd;
             float lo[3] = {gok ? gx : 3.0e38f, gok ? gy : 3.0e38f, gok ? gz : 3.0e38f};
