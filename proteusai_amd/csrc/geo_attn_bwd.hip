@@ -40,7 +40,8 @@ constexpr int GB_OWN     = GB_WAVES * 32;   // own tokens per workgroup
 constexpr int GB_BN      = 64;              // streamed tokens per tile
 constexpr int GB_D       = 64;
 constexpr int GB_LDR     = GB_D + 8;        // row stride of a row-major tile [token][d] (bf16 elements)
-constexpr int GB_LDT     = GB_BN + 8;       // row stride of a transposed tile [d][token]
+constexpr int GB_LDT     = GB_BN + 4;       // row stride of a transposed tile [d][token]: 34 dwords, so the 32 rows a
+                                            // half-wave reads 8 bytes from fall into 32 different bank pairs
 constexpr float LOG2E    = 1.4426950408889634f;
 
 struct __align__(16) BwdSmem {
