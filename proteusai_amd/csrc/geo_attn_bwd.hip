@@ -50,9 +50,11 @@ struct __align__(16) BwdSmem {
     uint16_t ta[GB_D * GB_LDT];      // first tensor transposed:  A operand of dQ^T / dK^T
     uint16_t tb[GB_D * GB_LDT];      // second tensor transposed (dO^T): A operand of dV^T (keys-own pass only)
     float    rx[GB_BN], ry[GB_BN], rz[GB_BN];   // coordinates of the other tokens
-    float    rl[GB_BN], rd[GB_BN];   // per other token: L*log2(e) if it is a usable query, 0 if a usable key, +inf if
-                                     // unusable (padded / out of range / empty row); D of a usable query, else 0
+    float    rl[GB_BN], rd[GB_BN];   // per other token that is a usable query: -L*log2(e) and D; -inf and 0 for an
+                                     // unusable one (padded / out of range / empty row).  When they are keys:
+                                     // rl = 0 for a usable key, -inf for an unusable one
     float    box[8];                 // bounding box of the usable other tokens of the tile: lo xyz, hi xyz
+    int      any_bad;                // the tile holds an unusable token
 };
 
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
@@ -112,6 +114,12 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         own_d  = own_use ? Dh[oc] : 0.f;
     }
     if (!own_use) own_l2 = INFINITY;
+    // Validity needs no select per pair: an unusable token's operands are zeros, so its S, dP and every
+    // product it is contracted in vanish; the exponent offset of an unusable QUERY is -inf (its L is -inf
+    // or garbage), which makes its P an exact 0.  An unusable KEY streamed past a query gets the offset
+    // -inf as well, but only in tiles that hold one (otherwise a query with a very negative L could
+    // overflow P for it, and inf * 0 is not 0).
+    const float own_off = -own_l2;
     const float ox = own_use ? cz[3 * oc] : 0.f, oy = own_use ? cz[3 * oc + 1] : 0.f, oz = own_use ? cz[3 * oc + 2] : 0.f;
     // bounding box of the wave's usable own tokens (for the far-tile test)
     float blo[3] = {own_use ? ox : 3.0e38f, own_use ? oy : 3.0e38f, own_use ? oz : 3.0e38f};
@@ -204,7 +212,8 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             if (!OWN_Q) gok = gok && (gl > -INFINITY);
             // an unusable token's coordinates, L and D may hold anything: zeros keep every product finite
             if (!gok) { gx = 0.f; gy = 0.f; gz = 0.f; gd = 0.f; }
-            gl = gok ? (OWN_Q ? 0.f : gl * LOG2E) : INFINITY;
+            gl = gok ? (OWN_Q ? 0.f : -gl * LOG2E) : -INFINITY;
+            const bool bad = __builtin_amdgcn_ballot_w64(!gok) != 0;
             sm.rx[tid] = gx; sm.ry[tid] = gy; sm.rz[tid] = gz;
             sm.rl[tid] = gl; sm.rd[tid] = gd;
             float lo[3] = {gok ? gx : 3.0e38f, gok ? gy : 3.0e38f, gok ? gz : 3.0e38f};
@@ -215,6 +224,7 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             if (tid == 0) {
 #pragma unroll
                 for (int c = 0; c < 3; ++c) { sm.box[c] = lo[c]; sm.box[3 + c] = hi[c]; }
+                sm.any_bad = bad ? 1 : 0;
             }
         }
     };
@@ -230,6 +240,7 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         // far-tile test: distance between the box of this wave's own tokens and the box of the tile's tokens.
         // Beyond `far2` the multiplier is 1 to fp32 rounding and its derivative terms vanish, so the geometry
         // is skipped for the whole tile (the legacy logits depend on rbf down to 0: always evaluated).
+        const bool any_bad = OWN_Q && sm.any_bad != 0;
         bool near = true;
         if (!LEGACY) {
             float g2 = 0.f;
@@ -263,8 +274,11 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int rb0 = mt * 32 + 8 * g + 4 * half;
-                    const float4 kl = *reinterpret_cast<const float4*>(&sm.rl[rb0]);
-                    const float ls[4] = {kl.x, kl.y, kl.z, kl.w};
+                    float ls[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (!OWN_Q || any_bad) {
+                        const float4 kl = *reinterpret_cast<const float4*>(&sm.rl[rb0]);
+                        ls[0] = kl.x; ls[1] = kl.y; ls[2] = kl.z; ls[3] = kl.w;
+                    }
                     float xs[4] = {0.f, 0.f, 0.f, 0.f}, ys[4] = {0.f, 0.f, 0.f, 0.f}, zs[4] = {0.f, 0.f, 0.f, 0.f};
                     float dds[4] = {0.f, 0.f, 0.f, 0.f};
                     if (NEAR) {
@@ -283,7 +297,7 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                     for (int v = 0; v < 4; ++v) {
                         const int r = 4 * g + v;
                         const float s  = sacc[r];
-                        const float off = -(ls[v] + own_l2);          // -(L log2e) of the pair's query, -inf if unusable
+                        const float off = OWN_Q ? (any_bad ? own_off + ls[v] : own_off) : ls[v];   // -(L log2e) of the pair's query, -inf if unusable
                         const float dd = OWN_Q ? own_d : dds[v];
                         if (!NEAR) {
                             const float p  = __builtin_amdgcn_exp2f(__builtin_fmaf(s, log2e_v, off));
