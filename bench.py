@@ -216,6 +216,35 @@ def main():
                          "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES},
         }
 
+        # ---- backward of the same shape (dQ, dK, dV, d sigma from the forward's O and L) ----
+        gq = torch.Generator().manual_seed(5)
+        dOb = (torch.randn(1, 8, 16384, 64, generator=gq) / 8).bfloat16().to(dev)
+        Dv = (O * dOb.float()).sum(-1).contiguous()
+        dQ_, dK_, dV_ = (torch.empty(1, 8, 16384, 64, device=dev) for _ in range(3))
+        dsg = torch.zeros(8, device=dev)
+
+        def bwd_step():
+            rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dOb.data_ptr(), acd.data_ptr(), sg.data_ptr(),
+                                          None, None, L.data_ptr(), Dv.data_ptr(), dQ_.data_ptr(), dK_.data_ptr(), dV_.data_ptr(),
+                                          dsg.data_ptr(), None, 1, 8, 16384, 64, 0.0, 1.0, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_geo_attn_bwd")
+        for _ in range(2):
+            bwd_step()
+        torch.cuda.synchronize()
+        bev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(5)]
+        for e0, e1 in bev:
+            e0.record()
+            bwd_step()
+            e1.record()
+        torch.cuda.synchronize()
+        b_ms = sum(e0.elapsed_time(e1) for e0, e1 in bev) / len(bev)
+        result["geo_attn_bwd"] = {
+            "workload": "geometric attention backward, same shape: dQ, dK, dV, d_sigma (two launches, S and dP recomputed in each)",
+            "ms": b_ms, "tflops_5_products": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12,
+            "tflops_issued_7_products": 14.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12, "dtype": "bf16",
+        }
+
     # ---------------- encoder forward, B=8, N=1024, 4 layers, bf16 weights, fp32 WE (configs[3]) ----------------
     if not args.no_encoder:
         import proteusai_amd as pa

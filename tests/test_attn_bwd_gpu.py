@@ -3,7 +3,7 @@ autograd function, against torch.autograd through the dense fp64 statement of th
 bf16-rounded inputs.
 
 Bar: the operands of every matrix product are bf16 (Q, K, V, dO, P, dS; the reference uses fp16), so each
-gradient tensor is compared in relative L2 norm: <= 2e-2 for dQ, dK, dV, d_sigma, d_beta."""
+gradient tensor is compared in relative L2 norm: <= 1e-2 for dQ, dK, dV, d_sigma, d_beta (measured: 2.4e-3)."""
 import numpy as np
 import pytest
 import torch
@@ -14,7 +14,7 @@ from proteusai_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-REL_L2_TOL = 2e-2
+REL_L2_TOL = 1e-2
 
 
 def rel_l2(a, b):

@@ -74,3 +74,32 @@ def test_cfg4_shape_bf16_and_padding_independence(gpu):
     valid = ~mask
     assert out.shape == (8, 1024, 20) and torch.isfinite(out[valid]).all()
     assert torch.equal(out[valid], out2[valid])
+
+
+def test_training_step_through_both_kernels(gpu):
+    # forward and backward of the whole stack on the HIP kernels (attention backward, wavenumber backward of the
+    # embedding), one SGD step, and the loss goes down
+    torch.manual_seed(1)
+    model = pa.ProteusEncoder(d_model=128, heads=2, layers=2, d_hidden=256).to(gpu)
+    model.wf_embedding.wavenumbers.requires_grad_(True)
+    g = torch.Generator().manual_seed(2)
+    coords = torch.stack([synth.random_walk_chain(120, g) for _ in range(2)]).to(gpu)
+    tokens = torch.randint(0, 33, (2, 120), generator=g).to(gpu)
+    labels = torch.randint(0, 20, (2, 120), generator=g).to(gpu)
+    mask = torch.zeros(2, 120, dtype=torch.bool, device=gpu)
+    mask[1, 90:] = True
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    losses = []
+    for _ in range(4):
+        opt.zero_grad()
+        logits = model(coords, tokens, mask)
+        loss = F.cross_entropy(logits[~mask], labels[~mask])
+        loss.backward()
+        for name, p in model.named_parameters():
+            if p.requires_grad and "beta_weights" not in name and "aa_magnitudes" not in name:
+                assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0]
+    assert model.layers[0].attn.spread_weights.grad.abs().sum() > 0
+    assert model.wf_embedding.wavenumbers.grad.abs().sum() > 0
