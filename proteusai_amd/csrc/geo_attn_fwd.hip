@@ -59,7 +59,8 @@ constexpr int GA_BM      = GA_WAVES * 32 * GA_QB;    // queries per workgroup
 constexpr int GA_BN      = 64;              // keys per tile
 constexpr int GA_D       = 64;              // head dim
 constexpr int GA_LDK     = GA_D + 8;        // LDS row stride of the K tile (bf16 elements)
-constexpr int GA_LDV     = GA_BN + 8;       // LDS row stride of the V^T tile
+constexpr int GA_LDV     = GA_BN + 4;       // LDS row stride of the V^T tile: 34 dwords, so the 32 rows a half-wave
+                                            // reads 8 bytes from fall into 32 different bank pairs
 constexpr int GA_LDG     = 40;              // LDS row stride of the key geometry tile (24 used)
 constexpr float LOG2E    = 1.4426950408889634f;
 // Largest squared distance (scaled units) of a workgroup's queries from their origin for
