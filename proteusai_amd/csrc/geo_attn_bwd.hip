@@ -252,19 +252,21 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             near = !(g2 > far2);             // (an empty box gives an infinite gap: far, and every P is 0 anyway)
         }
 
-#pragma unroll 1
-        for (int mt = 0; mt < 2; ++mt) {
-            // ---- S and dP of the 32 x 32 block: rows = other tokens, column = own token ----
-            floatx16 sacc, pacc;
+        // ---- S and dP of a 32 x 32 block: rows = other tokens, column = own token ----
+        auto score_mfma = [&](const int mt, floatx16& sa, floatx16& pa) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+            for (int r = 0; r < 16; ++r) { sa[r] = 0.f; pa[r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 const uint4 fa = *reinterpret_cast<const uint4*>(&sm.ra[(mt * 32 + col) * GB_LDR + ks * 16 + half * 8]);
                 const uint4 fb = *reinterpret_cast<const uint4*>(&sm.rb[(mt * 32 + col) * GB_LDR + ks * 16 + half * 8]);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), bs[ks], sacc, 0, 0, 0);
-                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), bp[ks], pacc, 0, 0, 0);
+                sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), bs[ks], sa, 0, 0, 0);
+                pa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), bp[ks], pa, 0, 0, 0);
             }
+        };
+        // The queries-own pass has the registers to issue the second block's matrix products before the
+        // first block's vector work, so they run under it; the keys-own pass takes the blocks one at a time.
+        auto process_block = [&](const int mt, const floatx16& sacc, const floatx16& pacc) {
             // ---- per pair: multiplier, P, dt, dS; accumulator register r is row 8*(r/4) + 4*half + (r%4).
             // Unusable tokens carry +inf in their exponent offset: P = exp2(-inf) = 0, and since their
             // operands and coordinates are zeros everything derived from P is an exact 0 as well. ----
@@ -357,6 +359,20 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                         acc_b[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb), __builtin_bit_cast(bf16x8, pb), acc_b[dt], 0, 0, 0);
                     }
                 }
+            }
+        };
+        if constexpr (OWN_Q) {
+            floatx16 sa[2], pa[2];
+            score_mfma(0, sa[0], pa[0]);
+            score_mfma(1, sa[1], pa[1]);
+            process_block(0, sa[0], pa[0]);
+            process_block(1, sa[1], pa[1]);
+        } else {
+#pragma unroll 1
+            for (int mt = 0; mt < 2; ++mt) {
+                floatx16 sa, pa;
+                score_mfma(mt, sa, pa);
+                process_block(mt, sa, pa);
             }
         }
     }
