@@ -264,7 +264,8 @@ const char* proteus_geo_attn_variant_name(int tuning);
  *       both in one stream, and the MFMAs with 32 v_exp_f32 in one stream;
  *       31..33: blocks/2 workgroups of 8 waves: waves 0-3 alone (four MFMAs per
  *       link), waves 4-7 alone (16 v_exp_f32 + 16 v_fmac_f32 per link), both kinds
- *       together (matrix and vector work in different waves of a SIMD)
+ *       together (matrix and vector work in different waves of a SIMD);
+ *       34: 64 chains of v_mul_f32 whose first source is a quad broadcast through DPP
  */
 int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
 

@@ -122,6 +122,30 @@ void valu_vector_operand_kernel(float* sink, int iters, float a, float b) {
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// 64 chains of v_mul_f32 whose first source goes through DPP (quad broadcast of one lane of a vector
+// register): a way to feed a wave-uniform factor without a scalar-register operand.
+__global__ __launch_bounds__(256)
+void valu_dpp_mul_kernel(float* sink, int iters, float a, float b) {
+    float x[64];
+#pragma unroll
+    for (int c = 0; c < 64; ++c) x[c] = 0.001f * (float)(threadIdx.x + c) + 0.25f;
+    float u = a + 1e-9f * (float)(threadIdx.x & 3) + b;
+#pragma unroll 1
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int c = 0; c < 64; c += 4) {
+            asm volatile("v_mul_f32_dpp %0, %1, %0 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(x[c]) : "v"(u));
+            asm volatile("v_mul_f32_dpp %0, %1, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(x[c + 1]) : "v"(u));
+            asm volatile("v_mul_f32_dpp %0, %1, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(x[c + 2]) : "v"(u));
+            asm volatile("v_mul_f32_dpp %0, %1, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(x[c + 3]) : "v"(u));
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 64; ++c) s += x[c];
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // The embedding kernel's inner step on register data: per wavenumber one v_mul_f32 with a scalar operand,
 // (TRANS: v_sin_f32 + v_cos_f32, else two more v_mul_f32), two v_fmac_f32 and two v_add_f32 on vector
 // operands, KT wavenumbers per step.  Instructions issued per lane and step: 7*KT.
@@ -345,13 +369,14 @@ extern "C" const char* proteus_strerror(int code) {
 extern "C" int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;
     if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return PROTEUS_ERR_BAD_SHAPE;
-    if (op < 0 || op > 33) return PROTEUS_ERR_BAD_TUNING;
+    if (op < 0 || op > 34) return PROTEUS_ERR_BAD_TUNING;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // a, b chosen so that the chains stay finite and are not constant-folded
     const float a = 0.999999f, b = 1e-7f;
 #define GO(OP_) hipLaunchKernelGGL((valu_rate_kernel<OP_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
 #define MIX(NT_, NF_) hipLaunchKernelGGL((valu_mix_kernel<NT_, NF_>), dim3(blocks), dim3(256), 0, st, sink, iters, a, b)
     switch (op) {
+        case 34: hipLaunchKernelGGL(valu_dpp_mul_kernel, dim3(blocks), dim3(256), 0, st, sink, iters, a, b); break;
         case 31: hipLaunchKernelGGL((mfma_cross_wave_kernel<0>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
         case 32: hipLaunchKernelGGL((mfma_cross_wave_kernel<1>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
         case 33: hipLaunchKernelGGL((mfma_cross_wave_kernel<2>), dim3((blocks + 1) / 2), dim3(512), 0, st, sink, iters, a, b); break;
