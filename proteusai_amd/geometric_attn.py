@@ -13,7 +13,7 @@ from . import _lib
 
 
 def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0,
-             betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0):
+             betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0, check_sigma: bool = True):
     """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None).
 
     Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569),
@@ -37,7 +37,8 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         raise AssertionError(f"number of spreads must be equal to nheads, not {tuple(sigma.shape)} and {H=}")
     if not Q.is_cuda:
         raise _lib.ProteusError("geo_attn needs tensors on the GPU (there is no CPU path)")
-    if not bool(torch.all(sigma > 0)):
+    # (reading the answer back synchronises with the device: callers whose sigma is positive by construction skip it)
+    if check_sigma and not bool(torch.all(sigma > 0)):
         raise AssertionError(f"spreads must be a tensor of positive, non-zero floats, not {sigma}")
     lib = _lib.load()
     dev = Q.device
@@ -120,9 +121,9 @@ class _geometric_attn(torch.autograd.Function):
     flows to the coordinates, as in the reference."""
 
     @staticmethod
-    def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf):
+    def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf, check_sigma=True):
         O, L = geo_attn(Q, K, V, coords, spreads, key_padding_mask, return_lse=True, betas=betas,
-                        min_rbf=min_rbf, max_rbf=max_rbf)
+                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma)
         ctx.save_for_backward(Q, K, V, O, L, coords, spreads, betas, key_padding_mask)
         ctx.min_rbf, ctx.max_rbf = min_rbf, max_rbf
         return O
@@ -133,10 +134,10 @@ class _geometric_attn(torch.autograd.Function):
         dQ, dK, dV, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
                                                         ctx.min_rbf, ctx.max_rbf)
         return (dQ.to(Q.dtype), dK.to(K.dtype), dV.to(V.dtype), None, d_sigma.to(spreads.dtype),
-                None if betas is None else d_beta.to(betas.dtype), None, None, None)
+                None if betas is None else d_beta.to(betas.dtype), None, None, None, None)
 
 
-def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00):
+def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True):
     """Same call as the reference's geometric_attn (geometric_attn.py:545-548).
 
     betas=None selects the README logits S*(1+RBF) (README.md:40; the rbf range must then be the full
@@ -145,7 +146,7 @@ def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00
     """
     if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
         raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
-    return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf)
+    return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads)
 
 
 class GeoAttention(nn.Module):
@@ -191,13 +192,31 @@ class GeoAttention(nn.Module):
         assert q.dim() == 3
         batch, N, d_model = q.shape
         assert d_model == self.d_model
-        Q = torch.matmul(q.unsqueeze(1), self.q_proj.unsqueeze(0)) + self.q_bias.unsqueeze(0).unsqueeze(2)
-        K = torch.matmul(k.unsqueeze(1), self.k_proj.unsqueeze(0)) + self.k_bias.unsqueeze(0).unsqueeze(2)
-        V = torch.matmul(v.unsqueeze(1), self.v_proj.unsqueeze(0)) + self.v_bias.unsqueeze(0).unsqueeze(2)
-        if self.legacy_logits:
-            out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf, max_rbf=self.max_rbf)
+        # Per-head projections x @ W_h + b_h (encoder.py:99-101) as plain GEMMs against the heads' weights laid
+        # side by side, [d_model, heads*d_k]: the broadcast batched matmul of the reference materialises the
+        # activations once per head.  Self-attention takes one GEMM for all three.
+        H, dk = self.heads, self.d_k
+
+        def flat(w):                       # [H, d_model, d_k] -> [d_model, H*d_k]
+            return w.permute(1, 0, 2).reshape(self.d_model, H * dk)
+
+        def heads_first(x):                # [Z, N, H*d_k] -> [Z, H, N, d_k]
+            return x.view(batch, N, H, dk).permute(0, 2, 1, 3)
+        if q is k and k is v:
+            w = torch.cat([flat(self.q_proj), flat(self.k_proj), flat(self.v_proj)], dim=1)
+            b = torch.cat([self.q_bias.reshape(-1), self.k_bias.reshape(-1), self.v_bias.reshape(-1)])
+            qkv = torch.addmm(b, q.reshape(batch * N, d_model), w).view(batch, N, 3, H * dk)
+            Q, K, V = heads_first(qkv[:, :, 0]), heads_first(qkv[:, :, 1]), heads_first(qkv[:, :, 2])
         else:
-            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask)
+            Q = heads_first(torch.addmm(self.q_bias.reshape(-1), q.reshape(batch * N, d_model), flat(self.q_proj)))
+            K = heads_first(torch.addmm(self.k_bias.reshape(-1), k.reshape(batch * N, d_model), flat(self.k_proj)))
+            V = heads_first(torch.addmm(self.v_bias.reshape(-1), v.reshape(batch * N, d_model), flat(self.v_proj)))
+        # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
+        if self.legacy_logits:
+            out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf,
+                                 max_rbf=self.max_rbf, check_spreads=False)
+        else:
+            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False)
         out = out.to(q.dtype)
         out = out.permute(0, 2, 3, 1)                    # batch x N x d_k x heads
         out = out.reshape(batch, N, self.d_model)
