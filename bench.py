@@ -273,6 +273,26 @@ def main():
                         "B=8 N=1024 lengths 128-1024, bf16 weights, fp32 WE (BASELINE.json configs[3])",
             "ms": e0.elapsed_time(e1) / 10, "valid_tokens": int(lens.sum()),
         }
+        # forward + backward of the same stack (cross-entropy on the unpadded tokens), no optimiser step
+        model.train()
+        labels = torch.randint(0, 20, (8, 1024), generator=g).to(dev)
+        keep = ~emask
+
+        def train_step():
+            model.zero_grad(set_to_none=True)
+            logits = model(ecoords, etokens, emask)
+            torch.nn.functional.cross_entropy(logits[keep].float(), labels[keep]).backward()
+        for _ in range(3):
+            train_step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            train_step()
+        e1.record()
+        torch.cuda.synchronize()
+        result["encoder_forward_backward"] = {"workload": "the same stack and batch, forward + backward (dropout 0)",
+                                              "ms": e0.elapsed_time(e1) / 10}
 
     # ---------------- CPU baseline: the tiled CPU PyTorch path on a bounded sample of observer rows ----------------
     if not args.no_cpu:
