@@ -53,8 +53,6 @@ struct __align__(16) BwdSmem {
     float    rl[GB_BN], rd[GB_BN];   // per other token that is a usable query: -L*log2(e) and D; -inf and 0 for an
                                      // unusable one (padded / out of range / empty row).  When they are keys:
                                      // rl = 0 for a usable key, -inf for an unusable one
-    float    box[8];                 // bounding box of the usable other tokens of the tile: lo xyz, hi xyz
-    int      any_bad;                // the tile holds an unusable token
 };
 
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
@@ -213,19 +211,8 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             // an unusable token's coordinates, L and D may hold anything: zeros keep every product finite
             if (!gok) { gx = 0.f; gy = 0.f; gz = 0.f; gd = 0.f; }
             gl = gok ? (OWN_Q ? 0.f : -gl * LOG2E) : -INFINITY;
-            const bool bad = __builtin_amdgcn_ballot_w64(!gok) != 0;
             sm.rx[tid] = gx; sm.ry[tid] = gy; sm.rz[tid] = gz;
             sm.rl[tid] = gl; sm.rd[tid] = gd;
-            float lo[3] = {gok ? gx : 3.0e38f, gok ? gy : 3.0e38f, gok ? gz : 3.0e38f};
-            float hi[3] = {gok ? gx : -3.0e38f, gok ? gy : -3.0e38f, gok ? gz : -3.0e38f};
-#pragma unroll
-            for (int c = 0; c < 3; ++c)
-                for (int off = 32; off > 0; off >>= 1) { lo[c] = fminf(lo[c], __shfl_xor(lo[c], off)); hi[c] = fmaxf(hi[c], __shfl_xor(hi[c], off)); }
-            if (tid == 0) {
-#pragma unroll
-                for (int c = 0; c < 3; ++c) { sm.box[c] = lo[c]; sm.box[3 + c] = hi[c]; }
-                sm.any_bad = bad ? 1 : 0;
-            }
         }
     };
 
@@ -237,19 +224,24 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         if (t + 1 < ntiles) load_tile((t + 1) * GB_BN);
         __syncthreads();
 
-        // far-tile test: distance between the box of this wave's own tokens and the box of the tile's tokens.
-        // Beyond `far2` the multiplier is 1 to fp32 rounding and its derivative terms vanish, so the geometry
-        // is skipped for the whole tile (the legacy logits depend on rbf down to 0: always evaluated).
-        const bool any_bad = OWN_Q && sm.any_bad != 0;
-        bool near = true;
-        if (!LEGACY) {
-            float g2 = 0.f;
+        // far-tile test: lane l takes the tile's token l and measures its distance to the box of this wave's own
+        // tokens.  If every usable token is beyond `far2` the multiplier is 1 to fp32 rounding and its derivative
+        // terms vanish, so the geometry is skipped for the whole tile (the legacy logits depend on rbf down to 0:
+        // always evaluated).
+        bool near = true, any_bad = false;
+        {
+            const bool usable = sm.rl[lane] > -INFINITY;
+            any_bad = OWN_Q && __builtin_amdgcn_ballot_w64(!usable) != 0;
+            if (!LEGACY) {
+                const float p[3] = {sm.rx[lane], sm.ry[lane], sm.rz[lane]};
+                float g2 = 0.f;
 #pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                const float gap = fmaxf(fmaxf(blo[c] - sm.box[3 + c], sm.box[c] - bhi[c]), 0.f);
-                g2 = __builtin_fmaf(gap, gap, g2);
+                for (int c = 0; c < 3; ++c) {
+                    const float gap = fmaxf(fmaxf(blo[c] - p[c], p[c] - bhi[c]), 0.f);
+                    g2 = __builtin_fmaf(gap, gap, g2);
+                }
+                near = __builtin_amdgcn_ballot_w64(usable && !(g2 > far2)) != 0;
             }
-            near = !(g2 > far2);             // (an empty box gives an infinite gap: far, and every P is 0 anyway)
         }
 
         // ---- S and dP of a 32 x 32 block: rows = other tokens, column = own token ----
