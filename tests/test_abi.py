@@ -222,3 +222,11 @@ def test_synthetic_inputs():
     assert torch.equal(c1, c2) and torch.equal(w1, w2)
     Q, K, V, c, sg, m = synth.attn_inputs(2, 2, 100, 64, 3, min_len=50)
     assert Q.dtype == torch.bfloat16 and m.shape == (2, 100) and (~m).sum(1).min() >= 50
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""

@@ -1,0 +1,96 @@
+"""Seeded random shapes, masks and scales through every kernel against its oracle: the fixed-shape tests
+cover the edge cases by hand, this file sweeps combinations nobody thought of (ragged N, odd K, head counts,
+batch sizes, mask densities, coordinate scales and offsets).  Same bars as the per-kernel test files."""
+import numpy as np
+import pytest
+import torch
+
+import proteusai_amd as pa
+from oracle import c_oracle, torch_oracle
+from proteusai_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    nb = np.linalg.norm(b)
+    return float(np.linalg.norm(a - b) / nb) if nb > 0 else float(np.linalg.norm(a - b))
+
+
+def chain(rng, Z, N, scale, offset):
+    steps = rng.normal(size=(Z, N, 3))
+    steps = 3.8 * steps / np.linalg.norm(steps, axis=-1, keepdims=True)
+    return torch.from_numpy((np.cumsum(steps, axis=1) * scale + offset).astype(np.float32))
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_wavefunction_embeddings(gpu, case):
+    rng = np.random.default_rng(1000 + case)
+    Z, N, K = int(rng.integers(1, 5)), int(rng.integers(1, 700)), int(rng.integers(1, 70))
+    coords = chain(rng, Z, N, float(rng.choice([0.3, 1.0, 4.0])), rng.normal(size=3) * float(rng.choice([0.0, 50.0, 2000.0])))
+    wn = torch.from_numpy(rng.uniform(0.05, 2.0, K).astype(np.float32) * rng.choice([-1.0, 1.0], K).astype(np.float32))
+    mask = torch.from_numpy(rng.random((Z, N)) < float(rng.choice([0.0, 0.1, 0.6])))
+    what = f"case {case}: Z={Z} N={N} K={K}"
+    got = pa.we_forward(coords.to(gpu), wn.to(gpu), mask.to(gpu))
+    ref = c_oracle.we(coords.numpy(), wn.numpy(), mask.numpy())
+    for g, r, name in zip(got, ref, ("out", "cos_sums", "sin_sums")):
+        g = g.cpu().numpy()
+        assert np.isfinite(g).all() and (g[mask.numpy()] == 0).all(), f"{what} {name}"
+        assert rel_l2(g, r) <= 1e-4, f"{what} {name}: {rel_l2(g, r):.3e}"
+    b = rng.normal(size=(Z, N, 3))
+    b = torch.from_numpy((b / np.linalg.norm(b, axis=-1, keepdims=True)).astype(np.float32))
+    cb = torch.from_numpy(rng.uniform(-2.0, 2.0, K).astype(np.float32))
+    got = pa.we_aniso_forward(coords.to(gpu), b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu))
+    ref = c_oracle.we_aniso(coords.numpy(), b.numpy(), cb.numpy(), wn.numpy(), mask.numpy())
+    for g, r, name in zip(got, ref, ("out", "d_cb", "d_k")):
+        g = g.cpu().numpy()
+        assert np.isfinite(g).all() and (g[mask.numpy()] == 0).all(), f"{what} aniso {name}"
+        assert rel_l2(g, r) <= 1e-4, f"{what} aniso {name}: {rel_l2(g, r):.3e}"
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_attention_forward_and_backward(gpu, case):
+    rng = np.random.default_rng(2000 + case)
+    Z, H, N = int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.integers(1, 400))
+    g = torch.Generator().manual_seed(3000 + case)
+    qs = float(rng.choice([0.5, 1.0, 2.0]))
+    Q = (torch.randn(Z, H, N, 64, generator=g) * qs).bfloat16()
+    K = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    dO = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    coords = chain(rng, Z, N, float(rng.choice([0.5, 1.0, 3.0])), rng.normal(size=3) * float(rng.choice([0.0, 100.0, 3000.0])))
+    sigma = torch.from_numpy(rng.uniform(1.0, 30.0, H).astype(np.float32))
+    mask = torch.from_numpy(rng.random((Z, N)) < float(rng.choice([0.0, 0.2, 0.7])))
+    legacy = case % 3 == 2
+    betas = torch.from_numpy(rng.uniform(0.1, 2.0, H).astype(np.float32)) if legacy else None
+    lo, hi = (0.02, 0.95) if legacy and case % 2 == 0 else (0.0, 1.0)
+    what = f"case {case}: Z={Z} H={H} N={N} legacy={legacy}"
+
+    q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
+    s = sigma.to(gpu).requires_grad_(True)
+    bt = None if betas is None else betas.to(gpu).requires_grad_(True)
+    O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi)
+    O.backward(dO.to(gpu).float())
+
+    rq, rk, rv = (t.double().requires_grad_(True) for t in (Q, K, V))
+    rs = sigma.double().requires_grad_(True)
+    rb = None if betas is None else betas.double().requires_grad_(True)
+    Oref = torch_oracle.geo_attn_autograd_torch(rq, rk, rv, coords, rs, mask, rb, lo, hi)
+    Oref.backward(dO.double())
+
+    Og = O.detach().cpu().double()
+    assert torch.isfinite(Og).all(), what
+    assert (Og - Oref.detach()).abs().max() <= 2e-2, f"{what}: O {(Og - Oref.detach()).abs().max():.3e}"
+    assert (Og[mask[:, None, :].expand(-1, H, -1)] == 0).all(), what
+    pairs = [(q.grad, rq.grad, "dQ"), (k.grad, rk.grad, "dK"), (v.grad, rv.grad, "dV"), (s.grad, rs.grad, "d_sigma")]
+    if legacy:
+        pairs.append((bt.grad, rb.grad, "d_beta"))
+    for gg, rr, name in pairs:
+        gg = gg.float().cpu().numpy()
+        assert np.isfinite(gg).all(), f"{what} {name}"
+        if np.linalg.norm(rr.numpy()) > 1e-9:
+            assert rel_l2(gg, rr.numpy()) <= 1e-2, f"{what} {name}: {rel_l2(gg, rr.numpy()):.3e}"
+        else:
+            assert np.abs(gg).max() <= 1e-6, f"{what} {name}"
