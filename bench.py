@@ -148,6 +148,32 @@ def main():
         "roofline": roofline,
     }
 
+    # ---------------- the same forward without the cos/sin sums (inference: nothing kept for a backward) ----------
+    def we_lean_step():
+        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(), None, out.data_ptr(), None, None,
+                                Z, N, K, args.we_tuning, stream)
+        if rc != 0:
+            _lib.check(rc, "proteus_we_fwd")
+    for _ in range(2):
+        we_lean_step()
+    torch.cuda.synchronize()
+    n_lean = max(5, args.steps // 2)
+    lev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_lean)]
+    for e0, e1 in lev:
+        e0.record()
+        we_lean_step()
+        e1.record()
+    torch.cuda.synchronize()
+    lean_ms = sum(e0.elapsed_time(e1) for e0, e1 in lev) / n_lean
+    # per unit: the phase product, v_sin, v_cos, one v_fmac and one v_add
+    lean_model_ms = W * (1.0 / rates["mul_s"] + 1.0 / rates["fmac_v"] + 1.0 / rates["add_v"] + 2.0 / r_trans) * 1e3
+    result["we_fwd_without_sums"] = {
+        "workload": "the headline shape with cos_sums = sin_sums = NULL (embedding only; not the headline metric, "
+                    "whose forward also returns the sums as the reference's does)",
+        "ms": lean_ms, "gpair_wavenumber_per_s": W / (lean_ms * 1e-3) / 1e9, "dtype": "f32",
+        "issue_model": {"model_ms": lean_model_ms, "frac": lean_model_ms / lean_ms},
+    }
+
     # ---------------- anisotropic (C-beta scaled) WE forward, same shape and chain ----------------
     if not args.no_aniso:
         g = torch.Generator().manual_seed(2)

@@ -78,7 +78,8 @@ const char* proteus_strerror(int code);
  *   coords       [Z,3,N] or [Z,N,3] f32, per coords_layout
  *   wavenumbers  [K] f32 (any sign)
  *   mask         [Z,N] u8, non-zero = padded; may be NULL (nothing padded)
- *   out          [Z,N,2K] f32     cos_sums, sin_sums  [Z,N,K] f32
+ *   out          [Z,N,2K] f32     cos_sums, sin_sums  [Z,N,K] f32, or BOTH NULL: then they are
+ *                not computed (inference: nothing is kept for the backward; a faster kernel)
  *   tuning       0 = automatic; otherwise a variant selector (see
  *                proteus_we_num_variants / proteus_we_variant_name)
  */

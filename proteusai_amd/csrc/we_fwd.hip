@@ -37,6 +37,10 @@ constexpr int WE_THREADS = WE_WAVES * 64;
 constexpr int WE_JB      = 256;   // sources staged per LDS block (one per thread)
 constexpr float WE_MAX_REV = 250.0f;
 
+// Value of the MAG template parameter for "weight 1/r, no cos/sin sums" (the caller passed no buffers for them:
+// inference, where nothing is kept for the backward; two of the four accumulations per unit fall away).
+constexpr int WE_MAG_NO_SUMS = -1;
+
 // Wavenumbers per phase batch of the inner loop (0: leave the order to the compiler).  On gfx950 a
 // vector instruction whose operands are all vector registers issues in about 2.4 clocks per wave once a
 // SIMD holds three or more waves, one with a scalar-register operand in 4, a transcendental in 8; an
@@ -78,7 +82,9 @@ __device__ __forceinline__ void stream_sources(const float4* s_keys, const int f
         const float e  = __builtin_fmaf(-r0, r0, r2);
         const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
         float m = inv, mr = 1.0f;
-        if (MAG == 1) {
+        if (MAG == WE_MAG_NO_SUMS) {
+            // weight 1/r, nothing kept for the backward
+        } else if (MAG == 1) {
             nzero += ok ? 0.0f : 1.0f;       // the r = 0 pair adds cos(0) = 1 to the cos sums: counted, removed at the end
         } else {
             // the r = 0 pair gets weight 0 in both sums
@@ -111,6 +117,7 @@ __device__ __forceinline__ void stream_sources(const float4* s_keys, const int f
                 const int t = t0 + u;
                 acc_oc[t] = __builtin_fmaf(cs[u], m, acc_oc[t]);
                 acc_os[t] = __builtin_fmaf(sn[u], m, acc_os[t]);
+                if (MAG == WE_MAG_NO_SUMS) continue;
                 if (MAG == 1) { acc_c[t] += cs[u]; acc_s[t] += sn[u]; }
                 else          { acc_c[t] = __builtin_fmaf(cs[u], mr, acc_c[t]); acc_s[t] = __builtin_fmaf(sn[u], mr, acc_s[t]); }
             }
@@ -213,6 +220,7 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
         }
 #pragma unroll
         for (int t = 0; t < KT; t += 4) {
+            if (MAG == WE_MAG_NO_SUMS) break;
             float4 c = make_float4((acc_c[t] - nzero) * keep, (acc_c[t + 1] - nzero) * keep,
                                    (acc_c[t + 2] - nzero) * keep, (acc_c[t + 3] - nzero) * keep);
             float4 s = make_float4(acc_s[t] * keep, acc_s[t + 1] * keep, acc_s[t + 2] * keep, acc_s[t + 3] * keep);
@@ -225,6 +233,7 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
             if (k0 + t < K) {
                 o[2 * t]     = acc_oc[t] * keep;
                 o[2 * t + 1] = acc_os[t] * keep;
+                if (MAG == WE_MAG_NO_SUMS) continue;
                 pc[t] = (acc_c[t] - nzero) * keep;
                 ps[t] = acc_s[t] * keep;
             }
@@ -378,7 +387,8 @@ extern "C" int proteus_we_fwd_check(const float* coords, int coords_layout,
                                     int Z, int N, int K, int tuning)
 {
     (void)mask;
-    if (!coords || !wavenumbers || !out || !cos_sums || !sin_sums) return PROTEUS_ERR_NULL_POINTER;
+    if (!coords || !wavenumbers || !out) return PROTEUS_ERR_NULL_POINTER;
+    if ((cos_sums == nullptr) != (sin_sums == nullptr)) return PROTEUS_ERR_NULL_POINTER;    // both or neither
     if (Z <= 0 || N <= 0 || K <= 0) return PROTEUS_ERR_BAD_SHAPE;
     if (N > PROTEUS_WE_MAX_N || K > PROTEUS_WE_MAX_K || Z > 65535) return PROTEUS_ERR_BAD_SHAPE;
     if (coords_layout != PROTEUS_COORDS_SOA && coords_layout != PROTEUS_COORDS_AOS) return PROTEUS_ERR_BAD_LAYOUT;
@@ -428,8 +438,10 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
             if (est < best * 0.999) { best = est; kt = ckt; split = csp; }
         }
     }
-#define WE_GO(KT_) (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st) \
-                          : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st))
+#define WE_GO(KT_) (!cos_sums ? (split ? launch<KT_, true, WE_MAG_NO_SUMS>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st) \
+                                      : launch<KT_, false, WE_MAG_NO_SUMS>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st)) \
+                    : (split ? launch<KT_, true>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st) \
+                             : launch<KT_, false>(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, fract, st)))
     switch (kt) {
         case 32: return WE_GO(32);
         case 16: return WE_GO(16);
@@ -456,6 +468,7 @@ extern "C" int proteus_we_legacy_fwd(const float* coords, int coords_layout,
     if (magnitude_type < 0 || magnitude_type > 3) return PROTEUS_ERR_UNSUPPORTED;
     if (magnitude_type == 1)
         return proteus_we_fwd(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 0, stream);
+    if (!cos_sums || !sin_sums) return PROTEUS_ERR_NULL_POINTER;      // the variant without sums exists for 1/r only
     const int rc = proteus_we_fwd_check(coords, coords_layout, wavenumbers, mask, out, cos_sums, sin_sums, Z, N, K, 0);
     if (rc != PROTEUS_OK) return rc;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);

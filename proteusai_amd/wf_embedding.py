@@ -13,9 +13,10 @@ from . import _lib
 from .cb_utils import get_coords
 
 
-def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: int = 1):
+def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: int = 1, need_sums: bool = True):
     """out, cos_sums, sin_sums = we_forward(coords [Z,N,3], wavenumbers [K], mask [Z,N] bool | None).
 
+    need_sums=False (weight 1/r only) skips the sums, which only the backward uses: returns (out, None, None).
     magnitude_type: the weight of a source at distance r, 0: 1, 1: 1/r (default), 2: 1/log2(r),
     3: 1/sqrt(r) (isotropic/cuda/wf_embedding_kernel.cu:192-206); the sums carry the weight times r.
 
@@ -43,8 +44,9 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
             raise ValueError(f"mask must be of shape ({Z}, {N}), not {tuple(mask.shape)}")
         m = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
     out = torch.empty(Z, N, 2 * K, dtype=torch.float32, device=dev)
-    cos_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev)
-    sin_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev)
+    need_sums = need_sums or magnitude_type != 1
+    cos_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev) if need_sums else None
+    sin_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev) if need_sums else None
     if Z == 0 or N == 0 or K == 0:
         return out, cos_sums, sin_sums
     with torch.cuda.device(dev):
@@ -52,7 +54,8 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
         if magnitude_type == 1:
             rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
                                     None if m is None else m.data_ptr(),
-                                    out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
+                                    out.data_ptr(), cos_sums.data_ptr() if need_sums else None,
+                                    sin_sums.data_ptr() if need_sums else None,
                                     Z, N, K, int(tuning), stream)
         else:
             rc = lib.proteus_we_legacy_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
@@ -74,8 +77,11 @@ class _wf_embedding(torch.autograd.Function):
             raise AssertionError("magnitude_type must be one of 0, 1, 2, 3")
         if dropout_p != 0.0:
             raise NotImplementedError("dropout_p != 0 is not implemented; the module always passes 0.0")
-        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type)
-        ctx.save_for_backward(cos_sums, sin_sums)
+        # the sums are what the backward for the wavenumbers consumes: without that gradient they are not computed
+        need = bool(ctx.needs_input_grad[1])
+        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type, need_sums=need)
+        if need:
+            ctx.save_for_backward(cos_sums, sin_sums)
         ctx.wn_dtype = wavenumbers.dtype
         return out
 

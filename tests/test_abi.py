@@ -46,6 +46,7 @@ def test_we_argument_validation_happens_before_any_hip_call():
     assert call() == 0
     for name in ("coords", "wn", "out", "cs", "ss"):
         assert call(**{name: None}) == -1
+    assert call(cs=None, ss=None) == 0                # both sums absent: the variant that does not compute them
     for name in ("Z", "N", "K"):
         assert call(**{name: 0}) == -2 and call(**{name: -3}) == -2
     assert call(N=(1 << 22) + 1) == -2 and call(K=4097) == -2
@@ -163,6 +164,8 @@ def test_operator_argument_errors_match_the_reference_surface():
     lib = _lib.load()
     assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, 0x1000, 0x1000, 0x1000, 1, 8, 4, 4, None) == -7
     assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, None, 0x1000, 0x1000, 1, 8, 4, 2, None) == -1
+    # the other source weights have no variant without the sums
+    assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, 0x1000, None, None, 1, 8, 4, 2, None) == -1
     Q = torch.randn(1, 2, 8, 64)
     with pytest.raises(AssertionError):
         pa.geo_attn(Q, Q[:, :, :4], Q, coords, torch.ones(2))

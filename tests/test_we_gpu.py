@@ -95,6 +95,20 @@ def test_every_variant_gives_the_same_answer(gpu):
         check(run_gpu(gpu, coords, wn, mask, tuning=t), coords, wn, mask, what=f"variant {name}")
 
 
+def test_without_sums_the_embedding_is_unchanged(gpu):
+    """cos_sums = sin_sums = NULL selects kernels that skip the two sums; `out` must not depend on that."""
+    for N, Z, d_model in ((600, 2, 160), (1500, 1, 512), (64, 3, 16)):
+        coords, wn = synth.we_inputs(N, seed=N, batch=Z, d_model=d_model)
+        g = torch.Generator().manual_seed(N)
+        mask = torch.rand(Z, N, generator=g) < 0.2
+        c, w, m = coords.to(gpu), wn.to(gpu), mask.to(gpu)
+        for t, name in enumerate(_lib.we_variants()):
+            full, cs, ss = pa.we_forward(c, w, m, tuning=t)
+            lean, none_c, none_s = pa.we_forward(c, w, m, tuning=t, need_sums=False)
+            assert none_c is None and none_s is None
+            assert torch.equal(full, lean), f"variant {name}, N={N}"
+
+
 def test_masks(gpu):
     N = 333
     coords, wn = synth.we_inputs(N, seed=5, batch=4, d_model=64)
