@@ -68,6 +68,9 @@ constexpr float LOG2E    = 1.4426950408889634f;
 constexpr float GA_MFMA_DIST_MAX_RHO2 = 1000.0f;
 // exp2(-d^2) < 2^-25 for scaled distances d > GA_FAR: s*(1+rbf) then rounds to s in fp32
 constexpr float GA_FAR = 5.0f;
+// Lazy softmax reference: a block re-bases when the sum of its 16 exponentials per lane passes 2^24 (log2 units)
+constexpr float GA_REBASE     = 20.0f;
+constexpr float GA_REBASE_SUM = 16777216.0f;
 
 // One staged key tile.  Two of them are kept so that the next tile can be written
 // while the current one is still being read (one barrier per tile).
@@ -309,17 +312,27 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         }
     }
 
+    // Online softmax with a LAZY reference: p = exp(s - m2) where m2 is the maximum the query had seen when
+    // it was last re-based, not the running maximum.  A block re-bases (exact maximum, rescale of O and l) only
+    // if a query has nothing accumulated yet or one of its exponentials passed 2^GA_REBASE; everywhere else
+    // no maximum is taken at all, and -m2 enters the score product itself as one more contraction slot
+    // (-m2 split exactly into three bf16 pieces against ones), so the accumulator times log2(e) is the exponent.
     floatx16 oacc[GA_QB][2];
-    float m_run[GA_QB], l_run[GA_QB];
+    float m2[GA_QB], l_run[GA_QB];
+    uint2 moff[GA_QB];           // B operand of the offset product: slots 0..2 = pieces of -m2 (half-wave 0 only)
 #pragma unroll
     for (int b = 0; b < GA_QB; ++b) {
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[b][dt][r] = 0.f;
-        m_run[b] = -INFINITY;    // running maximum of s (natural units), same in both half-waves
+        m2[b] = 0.f;             // reference of the exponentials (natural units), same in both half-waves
         l_run[b] = 0.f;          // this half-wave's part of the running sum
+        moff[b] = make_uint2(0u, 0u);
     }
+    const unsigned ones2 = 0x3f803f80u;      // bf16 (1, 1)
+    float log2e = LOG2E;                     // kept in a vector register: an all-register multiply issues faster
+    asm volatile("" : "+v"(log2e));
 
     // staging roles
     const int kp   = tid & 31;   // V: key pair
@@ -435,14 +448,18 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         return (rbf >= min_rbf && rbf <= max_rbf) ? t : -INFINITY;
     };
 
-    // multiplier, mask, online softmax of one 32-key x 32-query block; returns P^T packed for the two
+    // multiplier, mask, exponentials of one 32-key x 32-query block; returns P^T packed for the two
     // K=16 steps.  Accumulator register r of key block mt is key  mt*32 + 8*(r/4) + 4*half + (r%4).
+    // On entry sacc holds s (natural units) for a near block and s - m2 for a far one; it is turned into the
+    // exponent (s' - m2) log2(e) first.
     auto softmax_block = [&](const TileBuf& tb, const int mt, const int b, floatx16& sacc, const floatx16& dacc,
                              const bool has_masked, const bool near, uint4 (&pb)[2]) {
         if (near) {
+            const float mneg = -m2[b] * log2e;
             if (use_mfma_dist) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[r] = apply_rbf(sacc[r], __builtin_amdgcn_exp2f(dacc[r]));
+                for (int r = 0; r < 16; ++r)
+                    sacc[r] = __builtin_fmaf(apply_rbf(sacc[r], __builtin_amdgcn_exp2f(dacc[r])), log2e, mneg);
             } else {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
@@ -457,10 +474,13 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                     for (int v = 0; v < 4; ++v) {
                         const float dx = qx[b] - kxs[v], dy = qy[b] - kys[v], dz = qz[b] - kzs[v];
                         const float d2 = dx * dx + dy * dy + dz * dz;
-                        sacc[4 * g + v] = apply_rbf(sacc[4 * g + v], __builtin_amdgcn_exp2f(-d2));
+                        sacc[4 * g + v] = __builtin_fmaf(apply_rbf(sacc[4 * g + v], __builtin_amdgcn_exp2f(-d2)), log2e, mneg);
                     }
                 }
             }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] *= log2e;
         }
         if (has_masked) {
 #pragma unroll
@@ -469,55 +489,80 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 sacc[4 * g + 0] += bb.x; sacc[4 * g + 1] += bb.y; sacc[4 * g + 2] += bb.z; sacc[4 * g + 3] += bb.w;
             }
         }
-        float tmax = sacc[0];
+        float lsum = 0.f;
+        auto exponentials = [&]() {
+            lsum = 0.f;
 #pragma unroll
-        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
-        tmax = xhalf_max(tmax);
-
-        // online softmax: rescale only when some query's maximum moved
-        const float m_new = fmaxf(m_run[b], tmax);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run[b]) != 0) {
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f((m_run[b] - m_use) * LOG2E);   // m_run = -inf -> 0
+            for (int t = 0; t < 2; ++t) {
+                // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
+                float p[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    p[e] = __builtin_amdgcn_exp2f(sacc[8 * t + e]);
+                    lsum += p[e];
+                }
+                pb[t] = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+            }
+        };
+        exponentials();
+        // re-base where a query has nothing yet (first contact) or an exponential ran away; +inf is caught too
+        if (__builtin_amdgcn_ballot_w64(!(lsum <= GA_REBASE_SUM) || l_run[b] == 0.f) != 0) {
+            float tmax = sacc[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
+            tmax = xhalf_max(tmax);
+            const float l_tot = xhalf_sum(l_run[b]);
+            float delta = 0.f;                          // by how much this query's reference moves (log2 units)
+            if (tmax != -INFINITY && (l_tot == 0.f || tmax > GA_REBASE)) delta = tmax;
+            // a query without anything accumulated has nothing to rescale (and its delta may be hugely negative)
+            const float alpha = (l_tot == 0.f) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[b][dt][r] *= alpha;
             l_run[b] *= alpha;
-            m_run[b] = m_new;
-        }
-        const float mneg = -((m_run[b] == -INFINITY) ? 0.f : m_run[b]) * LOG2E;
-        float lsum = 0.f;
+            m2[b] = __builtin_fmaf(delta, 0.69314718055994531f, m2[b]);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
-            float p[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t + e], LOG2E, mneg));
-                lsum += p[e];
-            }
-            pb[t] = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+            for (int r = 0; r < 16; ++r) sacc[r] -= delta;
+            exponentials();
+            float oh, om, ol;
+            split3(-m2[b], oh, om, ol);
+            moff[b] = (half == 0) ? make_uint2(pack_bf16(oh, om), pack_bf16(ol, 0.f)) : make_uint2(0u, 0u);
         }
         l_run[b] += lsum;
     };
 
-    // one 32-key block of the staged tile against both query blocks
-    auto key_block = [&](const TileBuf& tb, const int mt, const bool has_masked, const bool near) {
+    // LDS -> register fragment loads, issued well ahead of the matrix instructions that consume them
+    auto load_kf = [&](const TileBuf& tb, const int mt, uint4 (&kf)[4]) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+            kf[ks] = *reinterpret_cast<const uint4*>(&tb.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
+    };
+    auto load_vf = [&](const TileBuf& tb, const int mt, const int t, uint4 (&vf)[2]) {
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+            const uint16_t* row = &tb.vt[(dt * 32 + col) * GA_LDV + mt * 32 + 16 * t + 4 * half];
+            const uint2 a0 = *reinterpret_cast<const uint2*>(row);
+            const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
+            vf[dt] = make_uint4(a0.x, a0.y, a1.x, a1.y);
+        }
+    };
+
+    // One 32-key block of the staged tile against both query blocks.  kf holds this block's K fragments on
+    // entry; if `more`, it is refilled with the next block's right after the score products have consumed it, so
+    // those reads (and the first V^T fragments) are in flight during the exponentials.
+    auto key_block = [&](const TileBuf& tb, const int mt, const bool has_masked, const bool near, uint4 (&kf)[4], const bool more) {
         floatx16 sacc[GA_QB];
-        {
-            uint4 kf[4];
+#pragma unroll
+        for (int b = 0; b < GA_QB; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[b][r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
-                kf[ks] = *reinterpret_cast<const uint4*>(&tb.k[(mt * 32 + col) * GA_LDK + ks * 16 + half * 8]);
-#pragma unroll
-            for (int b = 0; b < GA_QB; ++b) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[b][r] = 0.f;
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
-                    sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]), qreg[b][ks], sacc[b], 0, 0, 0);
-            }
+                sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]), qreg[b][ks], sacc[b], 0, 0, 0);
+            if (!near)      // s - m2 straight from the matrix cores: ones against the pieces of -m2
+                sacc[b] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, make_uint2(ones2, ones2)),
+                                                                   __builtin_bit_cast(shortx4, moff[b]), sacc[b], 0, 0, 0);
         }
         uint4 g0 = make_uint4(0, 0, 0, 0);
         uint2 g1 = make_uint2(0, 0);
@@ -526,9 +571,10 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
             g0 = *reinterpret_cast<const uint4*>(grow + 8 * half);
             g1 = *reinterpret_cast<const uint2*>(grow + 16 + 4 * half);
         }
+        (void)more;
+        uint4 pb[GA_QB][2];
 #pragma unroll
         for (int b = 0; b < GA_QB; ++b) {
-            uint4 pb[2];
             floatx16 dacc = {};
             if (near && use_mfma_dist) {
 #pragma unroll
@@ -536,18 +582,23 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                 dacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, g0), __builtin_bit_cast(bf16x8, gq0[b]), dacc, 0, 0, 0);
                 dacc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(shortx4, g1), __builtin_bit_cast(shortx4, gq1[b]), dacc, 0, 0, 0);
             }
-            softmax_block(tb, mt, b, sacc[b], dacc, has_masked, near, pb);
-    #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            softmax_block(tb, mt, b, sacc[b], dacc, has_masked, near, pb[b]);
+        }
+        // every V^T fragment read from LDS serves both query blocks
+        if (more) load_kf(tb, mt + 1, kf);
+        uint4 vf0[2], vf1[2];
+        load_vf(tb, mt, 0, vf0);
+        load_vf(tb, mt, 1, vf1);
 #pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
-                    const uint16_t* row = &tb.vt[(dt * 32 + col) * GA_LDV + mt * 32 + 16 * t + 4 * half];
-                    const uint2 a0 = *reinterpret_cast<const uint2*>(row);
-                    const uint2 a1 = *reinterpret_cast<const uint2*>(row + 8);
-                    const uint4 vf = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                    oacc[b][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pb[t]), oacc[b][dt], 0, 0, 0);
-                }
-            }
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int b = 0; b < GA_QB; ++b)
+                oacc[b][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf0[dt]), __builtin_bit_cast(bf16x8, pb[b][0]), oacc[b][dt], 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int b = 0; b < GA_QB; ++b)
+                oacc[b][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf1[dt]), __builtin_bit_cast(bf16x8, pb[b][1]), oacc[b][dt], 0, 0, 0);
     };
 
     // ---- key loop: tile t is computed from LDS while tile t+1 travels global -> registers -> the other LDS buffer ----
@@ -566,8 +617,10 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         const bool has_masked = tb.flags[0] != 0;
         const bool near       = LEGACY || tb.near[wave] == t + 1;
         if (has_valid) {
-            key_block(tb, 0, has_masked, near);
-            key_block(tb, 1, has_masked, near);
+            uint4 kf[4];
+            load_kf(tb, 0, kf);
+            key_block(tb, 0, has_masked, near, kf, true);
+            key_block(tb, 1, has_masked, near, kf, false);
         }
         if (t + 1 < ntiles) {
             store_tile(sm.tile[(t + 1) & 1], t + 1);
@@ -593,7 +646,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                                                 oacc[b][dt][4 * g + 2] * inv_l, oacc[b][dt][4 * g + 3] * inv_l);
                     *reinterpret_cast<float4*>(orow + dt * 32 + 8 * g + 4 * half) = v;
                 }
-            if (L && half == 0) L[(size_t)zh * N + q[b]] = row_ok ? m_run[b] + __logf(l_tot) : -INFINITY;
+            if (L && half == 0) L[(size_t)zh * N + q[b]] = row_ok ? m2[b] + __logf(l_tot) : -INFINITY;
         }
     }
 }

@@ -99,6 +99,39 @@ def test_large_logits(gpu):
     check(run_gpu(gpu, *a), *a, what="large logits")
 
 
+@pytest.mark.parametrize("profile", ["rising", "falling", "sawtooth", "late_spike", "very_negative_start", "masked_start"])
+@pytest.mark.parametrize("near", [False, True])
+def test_softmax_reference_is_rebased_when_the_scores_run_away(gpu, profile, near):
+    """Scores that climb, fall or jump by hundreds along the key axis: the kernel keeps a lazy softmax reference
+    (no running maximum) and must re-base it exactly when an exponential would run away, whatever the order."""
+    N, H = 640, 2
+    g = torch.Generator().manual_seed(11)
+    j = torch.arange(N, dtype=torch.float32)
+    ramp = {"rising": -60 + 120 * j / (N - 1),
+            "falling": 60 - 120 * j / (N - 1),
+            "sawtooth": 50 * ((j % 97) / 96.0 * 2 - 1) * (1 + j / N),
+            "late_spike": torch.where(j == N - 3, torch.tensor(150.0), -20 + 0 * j),
+            "very_negative_start": torch.where(j < 200, torch.tensor(-300.0), 5 * torch.sin(j)),
+            "masked_start": 10 * torch.cos(j)}[profile]
+    # s_ij = q_i . k_j / 8 with q = 8 on one axis and k_j = ramp_j there, plus small noise on the other axes
+    Q = 0.05 * torch.randn(1, H, N, 64, generator=g)
+    K = 0.05 * torch.randn(1, H, N, 64, generator=g)
+    Q[..., 0] = 8.0
+    K[..., 0] = ramp
+    Q, K = Q.bfloat16(), K.bfloat16()
+    V = torch.randn(1, H, N, 64, generator=g).bfloat16()
+    coords = synth.random_walk_chain(N, g)[None]
+    # near: every pair within reach of the multiplier (it then doubles the scores); far: none but the diagonal
+    sigma = torch.tensor([2000.0, 3000.0]) if near else torch.tensor([0.05, 0.08])
+    mask = None
+    if profile == "masked_start":
+        mask = torch.zeros(1, N, dtype=torch.bool)
+        mask[0, :130] = True
+        mask[0, 300:333] = True
+    a = (Q, K, V, coords, sigma, mask)
+    check(run_gpu(gpu, *a), *a, what=f"{profile}, near={near}")
+
+
 def test_flat_multiplier_equals_sdpa_on_gpu(gpu):
     # sigma -> infinity: multiplier == 2 -> torch SDPA with scale 2/sqrt(d), evaluated in fp32 on the same bf16 values
     Q, K, V, coords, _, _ = make(3, 2, 4, 777)
