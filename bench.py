@@ -21,6 +21,7 @@ if ROOT not in sys.path:
 # published MI355X peaks used as roofline denominators
 PEAK_FP32_VECTOR_TFLOPS = 157.3     # packed-FMA vector fp32
 PEAK_BF16_MFMA_TFLOPS = 2500.0      # dense bf16 matrix
+PEAK_HBM_GBS = 8000.0               # HBM3E
 H100_REFERENCE_GPW = 6.87194767e10 / 0.386 / 1e9   # README.md:34: 386 ms at this exact shape on an H100
 
 # HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), bytes
@@ -173,6 +174,37 @@ def main():
         "ms": lean_ms, "gpair_wavenumber_per_s": W / (lean_ms * 1e-3) / 1e9, "dtype": "f32",
         "issue_model": {"model_ms": lean_model_ms, "frac": lean_model_ms / lean_ms},
     }
+
+    # ---------------- WE backward (the reduction of dO against the sums), same shape: HBM-bound ----------------
+    dO = torch.randn(Z, N, 2 * K, device=dev)
+    dk = torch.empty(K, device=dev)
+    ws_bytes = lib.proteus_we_bwd_workspace_bytes(Z, N, K)
+    ws = torch.empty(ws_bytes // 4, device=dev)
+
+    def we_bwd_step():
+        rc = lib.proteus_we_bwd(dO.data_ptr(), cs.data_ptr(), ss.data_ptr(), dk.data_ptr(), ws.data_ptr(), ws_bytes,
+                                Z, N, K, stream)
+        if rc != 0:
+            _lib.check(rc, "proteus_we_bwd")
+    for _ in range(3):
+        we_bwd_step()
+    torch.cuda.synchronize()
+    bev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+    for e0, e1 in bev:
+        e0.record()
+        we_bwd_step()
+        e1.record()
+    torch.cuda.synchronize()
+    b_ms = sorted(e0.elapsed_time(e1) for e0, e1 in bev)[len(bev) // 2]
+    b_bytes = 16.0 * Z * N * K                       # dO (8) + cos_sums (4) + sin_sums (4) per (token, wavenumber)
+    result["we_bwd"] = {
+        "workload": "WE backward for the wavenumbers, dO [1,16384,512] against the saved sums, two launches",
+        "ms": b_ms, "dtype": "f32",
+        "roofline": {"kernel": "we_bwd_partial_kernel + we_bwd_final_kernel", "bound": "hbm",
+                     "achieved": b_bytes / (b_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": b_bytes / (b_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None},
+    }
+    del dO, ws
 
     # ---------------- anisotropic (C-beta scaled) WE forward, same shape and chain ----------------
     if not args.no_aniso:

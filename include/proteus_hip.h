@@ -154,6 +154,37 @@ int         proteus_we_aniso_num_variants(void);
 const char* proteus_we_aniso_variant_name(int tuning);
 
 /*
+ * Backward of the wavefunction embedding: the contraction of dO with what the
+ * forward kept.  Replaces the tensor expressions of
+ *   isotropic/cuda/wf_embedding.py:64-83
+ *     d_wavenumbers[k] = sum_{z,n} dO[z,n,2k+1] cos_sums[z,n,k] - dO[z,n,2k] sin_sums[z,n,k]
+ *   anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:65-79
+ *     g_cb[k] = sum_{z,n} dO[z,n,2k] d_cb[z,n,2k] + dO[z,n,2k+1] d_cb[z,n,2k+1]   (g_k likewise from d_k)
+ *
+ *   d_out [Z,N,2K] f32 (8-byte aligned); cos_sums, sin_sums [Z,N,K]; d_cb, d_k [Z,N,2K];
+ *   outputs [K] f32, fully overwritten.  In the anisotropic call a gradient that is not
+ *   wanted is skipped by passing NULL for both its partials and its output.
+ *   workspace: device memory of at least proteus_we_bwd_workspace_bytes(Z, N, K) bytes,
+ *   owned by the caller, overwritten; calls that share one workspace must not overlap.
+ *   Deterministic (no atomics); bound by HBM: 16 / 24 bytes per (token, wavenumber).
+ */
+size_t proteus_we_bwd_workspace_bytes(int Z, int N, int K);
+
+int proteus_we_bwd(const float* d_out, const float* cos_sums, const float* sin_sums,
+                   float* d_wavenumbers, float* workspace, size_t workspace_bytes,
+                   int Z, int N, int K, void* stream);
+int proteus_we_bwd_check(const float* d_out, const float* cos_sums, const float* sin_sums,
+                         const float* d_wavenumbers, const float* workspace, size_t workspace_bytes,
+                         int Z, int N, int K);
+
+int proteus_we_aniso_bwd(const float* d_out, const float* d_cb, const float* d_k,
+                         float* g_cb, float* g_k, float* workspace, size_t workspace_bytes,
+                         int Z, int N, int K, void* stream);
+int proteus_we_aniso_bwd_check(const float* d_out, const float* d_cb, const float* d_k,
+                               const float* g_cb, const float* g_k,
+                               const float* workspace, size_t workspace_bytes, int Z, int N, int K);
+
+/*
  * RBF-scaled geometric flash-attention forward.
  *
  * Replaces the Triton launch `_attn_fwd[grid](...)` made by

@@ -17,6 +17,7 @@ SYMBOLS = [
     "proteus_version", "proteus_strerror",
     "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_num_variants", "proteus_we_variant_name",
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
+    "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
     "proteus_geo_attn_bwd_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
@@ -60,6 +61,17 @@ def load():
     lib.proteus_we_aniso_num_variants.restype = ci
     lib.proteus_we_aniso_variant_name.restype = ctypes.c_char_p
     lib.proteus_we_aniso_variant_name.argtypes = [ci]
+    sz = ctypes.c_size_t
+    lib.proteus_we_bwd_workspace_bytes.restype = sz
+    lib.proteus_we_bwd_workspace_bytes.argtypes = [ci, ci, ci]
+    lib.proteus_we_bwd.restype = ci
+    lib.proteus_we_bwd.argtypes = [vp, vp, vp, vp, vp, sz, ci, ci, ci, vp]
+    lib.proteus_we_bwd_check.restype = ci
+    lib.proteus_we_bwd_check.argtypes = [vp, vp, vp, vp, vp, sz, ci, ci, ci]
+    lib.proteus_we_aniso_bwd.restype = ci
+    lib.proteus_we_aniso_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, ci, ci, ci, vp]
+    lib.proteus_we_aniso_bwd_check.restype = ci
+    lib.proteus_we_aniso_bwd_check.argtypes = [vp, vp, vp, vp, vp, vp, sz, ci, ci, ci]
     lib.proteus_geo_attn_fwd.restype = ci
     lib.proteus_geo_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     lib.proteus_geo_attn_legacy_fwd.restype = ci

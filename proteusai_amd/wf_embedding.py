@@ -4,7 +4,8 @@ Mirrors the reference's Python surface (paths under utils/model_utils/wf_embeddi
   wf_embedding(...) / _wf_embedding      isotropic/cuda/wf_embedding.py:18-83
   wf_embedding_learnCB(...)              anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:16-79
   WaveFunctionEmbedding                  wf_embedding.py:24-49
-plus `we_forward` / `we_aniso_forward`, which also return what the kernels save for the backward.
+plus `we_forward` / `we_aniso_forward`, which also return what the kernels save for the backward, and
+`we_backward` / `we_aniso_backward`, the reductions the two backward passes consist of.
 """
 import torch
 import torch.nn as nn
@@ -66,6 +67,49 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
     return out, cos_sums, sin_sums
 
 
+def _bwd_prepare(dO, *saved):
+    if not dO.is_cuda:
+        raise RuntimeError("the WE backward runs on the HIP kernels only: tensors must be on the GPU")
+    Z, N, K2 = dO.shape
+    ts = [dO.contiguous().float()] + [None if t is None else t.contiguous().float() for t in saved]
+    lib = _lib.load()
+    ws = torch.empty(max(1, lib.proteus_we_bwd_workspace_bytes(Z, N, K2 // 2) // 4), dtype=torch.float32, device=dO.device)
+    return lib, ts, ws, Z, N, K2 // 2, torch.cuda.current_stream(dO.device).cuda_stream
+
+
+def we_backward(dO, cos_sums, sin_sums):
+    """d_wavenumbers [K] = sum over tokens of dO_imag * cos_sums - dO_real * sin_sums
+    (isotropic/cuda/wf_embedding.py:75-81), as one streaming reduction on the GPU."""
+    lib, (g, c, s), ws, Z, N, K, stream = _bwd_prepare(dO, cos_sums, sin_sums)
+    dk = torch.empty(K, dtype=torch.float32, device=dO.device)
+    if Z == 0 or N == 0 or K == 0:
+        return dk.zero_()
+    with torch.cuda.device(dO.device):
+        rc = lib.proteus_we_bwd(g.data_ptr(), c.data_ptr(), s.data_ptr(), dk.data_ptr(), ws.data_ptr(), ws.numel() * 4,
+                                Z, N, K, stream)
+    _lib.check(rc, "proteus_we_bwd")
+    return dk
+
+
+def we_aniso_backward(dO, d_cb=None, d_k=None):
+    """g_cb, g_k [K]: dO contracted with the saved per-token partials over tokens and over each (cos, sin) pair
+    (anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:65-79).  A partial passed as None is
+    skipped and its gradient returned as None."""
+    if d_cb is None and d_k is None:
+        return None, None
+    lib, (g, a, b), ws, Z, N, K, stream = _bwd_prepare(dO, d_cb, d_k)
+    g_cb = None if a is None else torch.empty(K, dtype=torch.float32, device=dO.device)
+    g_k = None if b is None else torch.empty(K, dtype=torch.float32, device=dO.device)
+    if Z == 0 or N == 0 or K == 0:
+        return (None if g_cb is None else g_cb.zero_()), (None if g_k is None else g_k.zero_())
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(dO.device):
+        rc = lib.proteus_we_aniso_bwd(g.data_ptr(), ptr(a), ptr(b), ptr(g_cb), ptr(g_k), ws.data_ptr(), ws.numel() * 4,
+                                      Z, N, K, stream)
+    _lib.check(rc, "proteus_we_aniso_bwd")
+    return g_cb, g_k
+
+
 class _wf_embedding(torch.autograd.Function):
     """Forward on the HIP kernel; analytical O(N K) backward for the wavenumbers
     (isotropic/cuda/wf_embedding.py:64-83).  No gradient flows to coords, as in
@@ -88,9 +132,7 @@ class _wf_embedding(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dO):
         cos_sums, sin_sums = ctx.saved_tensors
-        real_dO = dO[:, :, 0::2]
-        imag_dO = dO[:, :, 1::2]
-        dk = ((imag_dO * cos_sums) - (real_dO * sin_sums)).sum(dim=(0, 1))
+        dk = we_backward(dO, cos_sums, sin_sums)
         return None, dk.to(ctx.wn_dtype), None, None, None
 
 
@@ -153,17 +195,17 @@ class _wf_embedding_learnCB(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask):
         out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask)
-        ctx.save_for_backward(d_cb.to(cb_magnitudes.dtype), d_k.to(wavenumbers.dtype))
+        ctx.save_for_backward(d_cb, d_k)
+        ctx.dtypes = (cb_magnitudes.dtype, wavenumbers.dtype)
         return out.to(coordsA.dtype)
 
     @staticmethod
     def backward(ctx, dO):
         d_cb, d_k = ctx.saved_tensors
-        g_cb = (dO * d_cb).sum(dim=(0, 1))
-        g_cb = g_cb[0::2] + g_cb[1::2]
-        g_k = (dO * d_k).sum(dim=(0, 1))
-        g_k = g_k[0::2] + g_k[1::2]
-        return None, None, g_cb, g_k, None
+        g_cb, g_k = we_aniso_backward(dO, d_cb if ctx.needs_input_grad[2] else None,
+                                      d_k if ctx.needs_input_grad[3] else None)
+        return (None, None, None if g_cb is None else g_cb.to(ctx.dtypes[0]),
+                None if g_k is None else g_k.to(ctx.dtypes[1]), None)
 
 
 def wf_embedding_learnCB(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None):

@@ -233,3 +233,31 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_we_backward_argument_validation_happens_before_any_hip_call():
+    lib = _lib.load()
+    p = 0x1000
+    need = lib.proteus_we_bwd_workspace_bytes(2, 100, 16)
+    assert need >= 2 * 16 * 4 and lib.proteus_we_bwd_workspace_bytes(0, 100, 16) == 0
+    # the workspace grows with the rows only up to a fixed number of slabs
+    assert lib.proteus_we_bwd_workspace_bytes(1, 1 << 22, 16) == lib.proteus_we_bwd_workspace_bytes(1, 1 << 20, 16)
+    ok = lib.proteus_we_bwd_check(p, p, p, p, p, need, 2, 100, 16)
+    assert ok == 0
+    assert lib.proteus_we_bwd_check(None, p, p, p, p, need, 2, 100, 16) == -1
+    assert lib.proteus_we_bwd_check(p, None, p, p, p, need, 2, 100, 16) == -1
+    assert lib.proteus_we_bwd_check(p, p, p, None, p, need, 2, 100, 16) == -1
+    assert lib.proteus_we_bwd_check(p, p, p, p, None, need, 2, 100, 16) == -1
+    assert lib.proteus_we_bwd_check(p, p, p, p, p, need - 1, 2, 100, 16) == -2
+    assert lib.proteus_we_bwd_check(p, p, p, p, p, need, 0, 100, 16) == -2
+    assert lib.proteus_we_bwd_check(p, p, p, p, p, need, 2, 100, 4097) == -2
+    assert lib.proteus_we_bwd_check(p + 4, p, p, p, p, need, 2, 100, 16) == -5
+    assert lib.proteus_we_bwd(None, p, p, p, p, need, 2, 100, 16, None) == -1
+    # anisotropic: each gradient comes with its partials or not at all; at least one is wanted
+    assert lib.proteus_we_aniso_bwd_check(p, p, p, p, p, p, need, 2, 100, 16) == 0
+    assert lib.proteus_we_aniso_bwd_check(p, p, None, p, None, p, need, 2, 100, 16) == 0
+    assert lib.proteus_we_aniso_bwd_check(p, None, p, None, p, p, need, 2, 100, 16) == 0
+    assert lib.proteus_we_aniso_bwd_check(p, p, None, p, p, p, need, 2, 100, 16) == -1
+    assert lib.proteus_we_aniso_bwd_check(p, None, None, None, None, p, need, 2, 100, 16) == -1
+    assert lib.proteus_we_aniso_bwd_check(p, p, p, p, p, p, need - 4, 2, 100, 16) == -2
+    assert lib.proteus_we_aniso_bwd(p, p, p, p, p, None, need, 2, 100, 16, None) == -1

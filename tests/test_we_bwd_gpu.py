@@ -1,0 +1,113 @@
+"""GPU parity tests of the WE backward reductions (through the C ABI) against the tensor expressions of
+the reference's backward passes, evaluated in float64:
+  isotropic   isotropic/cuda/wf_embedding.py:75-81
+  anisotropic anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:70-77
+Bar: relative L2 error <= 1e-5 (fp32 accumulation over up to 10^5 rows in a different order)."""
+import numpy as np
+import pytest
+import torch
+
+import proteusai_amd as pa
+from proteusai_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-5
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+def iso_reference(dO, c, s):
+    dO, c, s = dO.double(), c.double(), s.double()
+    return ((dO[:, :, 1::2] * c) - (dO[:, :, 0::2] * s)).sum(dim=(0, 1))
+
+
+def aniso_reference(dO, a):
+    t = (dO.double() * a.double()).sum(dim=(0, 1))
+    return t[0::2] + t[1::2]
+
+
+SHAPES = [(1, 1, 1), (1, 5, 7), (2, 33, 64), (3, 100, 256), (1, 9000, 3), (2, 4500, 300), (1, 2048, 513), (4, 257, 40)]
+
+
+@pytest.mark.parametrize("Z,N,K", SHAPES)
+def test_isotropic_reduction(gpu, Z, N, K):
+    g = torch.Generator().manual_seed(Z * 1000 + N + K)
+    dO = torch.randn(Z, N, 2 * K, generator=g)
+    c = torch.randn(Z, N, K, generator=g) * 3
+    s = torch.randn(Z, N, K, generator=g) * 3
+    got = pa.we_backward(dO.to(gpu), c.to(gpu), s.to(gpu)).cpu()
+    assert got.shape == (K,)
+    assert rel_l2(got.numpy(), iso_reference(dO, c, s).numpy()) <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("Z,N,K", SHAPES)
+def test_anisotropic_reduction(gpu, Z, N, K):
+    g = torch.Generator().manual_seed(Z * 1000 + N + K + 1)
+    dO = torch.randn(Z, N, 2 * K, generator=g)
+    a = torch.randn(Z, N, 2 * K, generator=g)
+    b = torch.randn(Z, N, 2 * K, generator=g)
+    g_cb, g_k = pa.we_aniso_backward(dO.to(gpu), a.to(gpu), b.to(gpu))
+    assert rel_l2(g_cb.cpu().numpy(), aniso_reference(dO, a).numpy()) <= REL_L2_TOL
+    assert rel_l2(g_k.cpu().numpy(), aniso_reference(dO, b).numpy()) <= REL_L2_TOL
+    # either gradient alone: the other is skipped, the one asked for is bit-identical
+    only_cb, none_k = pa.we_aniso_backward(dO.to(gpu), a.to(gpu), None)
+    none_cb, only_k = pa.we_aniso_backward(dO.to(gpu), None, b.to(gpu))
+    assert none_k is None and none_cb is None
+    assert torch.equal(only_cb, g_cb) and torch.equal(only_k, g_k)
+
+
+def test_deterministic_and_workspace_canaries(gpu):
+    """Two calls give identical bits; nothing is written beyond the stated workspace size or the K outputs."""
+    lib = _lib.load()
+    Z, N, K = 2, 3000, 129
+    g = torch.Generator().manual_seed(5)
+    dO = torch.randn(Z, N, 2 * K, generator=g).to(gpu)
+    c = torch.randn(Z, N, K, generator=g).to(gpu)
+    s = torch.randn(Z, N, K, generator=g).to(gpu)
+    need = lib.proteus_we_bwd_workspace_bytes(Z, N, K)
+    assert need > 0 and need % 4 == 0
+    ws = torch.full((need // 4 + 64,), 7.5, device=gpu)
+    out = torch.full((K + 64,), -3.25, device=gpu)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.proteus_we_bwd(dO.data_ptr(), c.data_ptr(), s.data_ptr(), out.data_ptr(), ws.data_ptr(), need, Z, N, K, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert (ws[need // 4:] == 7.5).all() and (out[K:] == -3.25).all()
+    first = out[:K].clone()
+    rc = lib.proteus_we_bwd(dO.data_ptr(), c.data_ptr(), s.data_ptr(), out.data_ptr(), ws.data_ptr(), need, Z, N, K, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(first, out[:K])
+    assert rel_l2(first.cpu().numpy(), iso_reference(dO.cpu(), c.cpu(), s.cpu()).numpy()) <= REL_L2_TOL
+    # a workspace that is too small is refused before anything is launched
+    assert lib.proteus_we_bwd(dO.data_ptr(), c.data_ptr(), s.data_ptr(), out.data_ptr(), ws.data_ptr(), need - 4, Z, N, K, stream) == -2
+
+
+def test_gradients_through_the_operators(gpu):
+    """d(loss)/d(wavenumbers) and d(loss)/d(cb_magnitudes) from the autograd Functions equal the expressions
+    evaluated on what the forward kernels saved."""
+    from proteusai_amd import synth
+    coords, wn = synth.we_inputs(300, seed=9, batch=2, d_model=96)
+    g = torch.Generator().manual_seed(9)
+    mask = torch.rand(2, 300, generator=g) < 0.15
+    w = wn.to(gpu).requires_grad_(True)
+    out = pa.wf_embedding(coords.to(gpu), w, mask=mask.to(gpu))
+    dO = torch.randn(out.shape, generator=g).to(gpu)
+    out.backward(dO)
+    _, cs, ss = pa.we_forward(coords.to(gpu), wn.to(gpu), mask.to(gpu))
+    assert rel_l2(w.grad.cpu().numpy(), iso_reference(dO.cpu(), cs.cpu(), ss.cpu()).numpy()) <= REL_L2_TOL
+
+    cb_dir = torch.randn(2, 300, 3, generator=g)
+    cb_dir = cb_dir / cb_dir.norm(dim=-1, keepdim=True)
+    cbm = (0.5 + torch.rand(48, generator=g)).to(gpu).requires_grad_(True)
+    w2 = wn.to(gpu).requires_grad_(True)
+    out = pa.wf_embedding_learnCB(coords.to(gpu), cb_dir.to(gpu), cbm, w2, mask.to(gpu))
+    dO = torch.randn(out.shape, generator=g).to(gpu)
+    out.backward(dO)
+    _, d_cb, d_k = pa.we_aniso_forward(coords.to(gpu), cb_dir.to(gpu), cbm.detach(), wn.to(gpu), mask.to(gpu))
+    assert rel_l2(cbm.grad.cpu().numpy(), aniso_reference(dO.cpu(), d_cb.cpu()).numpy()) <= REL_L2_TOL
+    assert rel_l2(w2.grad.cpu().numpy(), aniso_reference(dO.cpu(), d_k.cpu()).numpy()) <= REL_L2_TOL
