@@ -54,8 +54,8 @@ typedef unsigned uint4v __attribute__((ext_vector_type(4)));
 
 constexpr int GA_WAVES   = 4;
 constexpr int GA_THREADS = GA_WAVES * 64;
-constexpr int GA_QB      = 2;                        // 32-query blocks per wave
-constexpr int GA_BM      = GA_WAVES * 32 * GA_QB;    // queries per workgroup
+// 32-query blocks per wave: 2 (256 queries per workgroup; every LDS fragment serves both blocks), or 1 for
+// grids that would otherwise leave half of the wave slots empty
 constexpr int GA_BN      = 64;              // keys per tile
 constexpr int GA_D       = 64;              // head dim
 constexpr int GA_LDK     = GA_D + 8;        // LDS row stride of the K tile (bf16 elements)
@@ -125,7 +125,7 @@ __device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
 // LEGACY selects the logits of the reference's Triton kernel instead of the README multiplier:
 //   s = S + beta_h * (2 (rbf - min_rbf)/(max_rbf - min_rbf) - 1) * |S|, pairs with rbf outside [min_rbf, max_rbf] masked
 //   (old/old_scripts/attn/geometric_attn.py:193-201).
-template <bool DIST_VALU, bool LEGACY>
+template <bool DIST_VALU, bool LEGACY, int GA_QB>
 __global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                          const uint16_t* __restrict__ V, const float* __restrict__ coords,
@@ -181,6 +181,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     __syncthreads();
 
     // ---- this lane's queries: one per block ----
+    constexpr int GA_BM = GA_WAVES * 32 * GA_QB;          // queries per workgroup
     const int qbase = qt * GA_BM + wave * (32 * GA_QB);
     int   q[GA_QB];
     bool  q_in[GA_QB], q_ok[GA_QB];
@@ -652,7 +653,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 }
 
 struct GaVariant { const char* name; };
-const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"} };
+const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -680,23 +681,40 @@ extern "C" int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, 
 }
 
 namespace {
+template <bool LEGACY, int QB>
+int launch_attn_qb(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                   const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int dist,
+                   const float* beta, float min_rbf, float max_rbf, hipStream_t st)
+{
+    constexpr int BM = GA_WAVES * 32 * QB;
+    const int n_qtiles = (N + BM - 1) / BM;
+    const int ZH = Z * H;
+    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
+    // dist 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
+    // 1 / 2: force the matrix-core / vector-ALU path everywhere
+    if (dist != 2)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 1 ? 1 : 0, beta, min_rbf, max_rbf);
+    if (dist != 1)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 2 ? 1 : 0, beta, min_rbf, max_rbf);
+    return (int)hipGetLastError();
+}
+
 template <bool LEGACY>
 int launch_attn(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                 const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
                 const float* beta, float min_rbf, float max_rbf, hipStream_t st)
 {
-    const int n_qtiles = (N + GA_BM - 1) / GA_BM;
-    const int ZH = Z * H;
-    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
-    // tuning 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
-    // 1 / 2: force the matrix-core / vector-ALU path everywhere
-    if (tuning != 2)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 1 ? 1 : 0, beta, min_rbf, max_rbf);
-    if (tuning != 1)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, tuning == 2 ? 1 : 0, beta, min_rbf, max_rbf);
-    return (int)hipGetLastError();
+    // Two query blocks per wave unless that leaves at most one workgroup per compute unit (256 of them on
+    // this chip, two workgroups each): then one block per wave doubles the waves in flight.
+    const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
+    bool one_block = wgs2 <= 256;
+    int dist = tuning;
+    if (tuning == 3) { one_block = true;  dist = 0; }
+    if (tuning == 4) { one_block = false; dist = 0; }
+    return one_block ? launch_attn_qb<LEGACY, 1>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, st)
+                     : launch_attn_qb<LEGACY, 2>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, st);
 }
 }  // namespace
 
@@ -724,7 +742,7 @@ extern "C" int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K,
     if (!beta) return PROTEUS_ERR_NULL_POINTER;
     if (!(max_rbf > min_rbf)) return PROTEUS_ERR_BAD_SHAPE;
     // a pair mask makes the result sensitive to the last bits of the rbf: use direct distances then
-    if (tuning == 0 && (min_rbf > 0.f || max_rbf < 1.f)) tuning = 2;
+    if ((tuning == 0 || tuning >= 3) && (min_rbf > 0.f || max_rbf < 1.f)) tuning = 2;
     return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf,
                              reinterpret_cast<hipStream_t>(stream));
 }

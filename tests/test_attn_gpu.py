@@ -132,6 +132,17 @@ def test_softmax_reference_is_rebased_when_the_scores_run_away(gpu, profile, nea
     check(run_gpu(gpu, *a), *a, what=f"{profile}, near={near}")
 
 
+def test_every_variant_matches_the_oracle(gpu):
+    """Distance path (matrix cores / vector ALU) and query blocks per wave (1 / 2) are tuning choices, not semantics."""
+    a = make(21, 2, 3, 700, maskfrac=0.1, tail=True)
+    Q, K, V, coords, sigma, mask = a
+    for t, name in enumerate(_lib.geo_attn_variants()):
+        O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu),
+                           return_lse=True, tuning=t)
+        torch.cuda.synchronize()
+        check((O.cpu().numpy(), L.cpu().numpy()), *a, what=f"variant {name}")
+
+
 def test_flat_multiplier_equals_sdpa_on_gpu(gpu):
     # sigma -> infinity: multiplier == 2 -> torch SDPA with scale 2/sqrt(d), evaluated in fp32 on the same bf16 values
     Q, K, V, coords, _, _ = make(3, 2, 4, 777)
