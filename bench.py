@@ -80,7 +80,8 @@ def main():
                     help="also launch a 256 MiB device copy, so a rocprofv3 --pmc run of this command holds a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (rows shard trivially, see DESIGN.md); "
+        print("bench.py measures one GPU: this build has no multi-GPU path (observer rows and (batch, head) pairs are "
+              "independent, so the work shards without any exchange); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
