@@ -265,6 +265,47 @@ int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint1
                                const float* d_sigma, const float* d_beta,
                                int Z, int H, int N, int d_head, float min_rbf, float max_rbf);
 
+/*
+ * The same forward and backward on tensors that are not contiguous [Z,H,N,64].
+ *
+ * The reference's Triton launches take every tensor's strides
+ * (old/old_scripts/attn/geometric_attn.py:588-599, :627-648); these entry
+ * points take the (batch, head, token) strides in ELEMENTS, the head dimension
+ * being contiguous:
+ *   forward   strides[12] : Q, K, V, O
+ *   backward  strides[21] : Q, K, V, dO, dQ, dK, dV
+ * so that slices of a fused [Z,N,3,H,64] projection are read in place and O or the
+ * gradients are written in the memory order their consumer wants (e.g. [Z,N,H,64]).
+ * Per tensor: token stride >= 64, no negative stride, batch / head stride 0 only for
+ * Z == 1 / H == 1 (else PROTEUS_ERR_BAD_LAYOUT); every stride a multiple of 16 bytes
+ * (PROTEUS_ERR_BAD_ALIGNMENT); N * token stride below 2^31 bytes (forward) or
+ * 2^30 elements (backward) (PROTEUS_ERR_BAD_SHAPE).  coords, sigma, beta, the mask, L and D stay
+ * contiguous.  Everything else is as for proteus_geo_attn_fwd / proteus_geo_attn_bwd.
+ */
+int proteus_geo_attn_fwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                 const int64_t* strides,
+                                 const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                 float* O, float* L,
+                                 int Z, int H, int N, int d_head, int tuning, void* stream);
+int proteus_geo_attn_fwd_strided_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                       const int64_t* strides,
+                                       const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                       const float* O, const float* L,
+                                       int Z, int H, int N, int d_head, int tuning);
+int proteus_geo_attn_bwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                 const int64_t* strides,
+                                 const float* coords, const float* sigma, const float* beta,
+                                 const uint8_t* key_pad_mask, const float* L, const float* D,
+                                 float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
+                                 int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream);
+int proteus_geo_attn_bwd_strided_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                       const int64_t* strides,
+                                       const float* coords, const float* sigma, const float* beta,
+                                       const uint8_t* key_pad_mask, const float* L, const float* D,
+                                       const float* dQ, const float* dK, const float* dV,
+                                       const float* d_sigma, const float* d_beta,
+                                       int Z, int H, int N, int d_head, float min_rbf, float max_rbf);
+
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);
 

@@ -19,7 +19,8 @@ SYMBOLS = [
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
     "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
-    "proteus_geo_attn_bwd_check", "proteus_geo_attn_num_variants",
+    "proteus_geo_attn_bwd_check", "proteus_geo_attn_fwd_strided", "proteus_geo_attn_fwd_strided_check",
+    "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_probe_valu_rate", "proteus_probe_sincos",
 ]
@@ -82,6 +83,15 @@ def load():
     lib.proteus_geo_attn_bwd.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf, vp]
     lib.proteus_geo_attn_bwd_check.restype = ci
     lib.proteus_geo_attn_bwd_check.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf]
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    lib.proteus_geo_attn_fwd_strided.restype = ci
+    lib.proteus_geo_attn_fwd_strided.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.proteus_geo_attn_fwd_strided_check.restype = ci
+    lib.proteus_geo_attn_fwd_strided_check.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
+    lib.proteus_geo_attn_bwd_strided.restype = ci
+    lib.proteus_geo_attn_bwd_strided.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, vp]
+    lib.proteus_geo_attn_bwd_strided_check.restype = ci
+    lib.proteus_geo_attn_bwd_strided_check.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf]
     lib.proteus_geo_attn_fwd_check.restype = ci
     lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_num_variants.restype = ci
@@ -119,3 +129,11 @@ def we_aniso_variants():
 def geo_attn_variants():
     lib = load()
     return [lib.proteus_geo_attn_variant_name(i).decode() for i in range(lib.proteus_geo_attn_num_variants())]
+
+
+def stride_array(*tensors):
+    """(batch, head, token) element strides of [Z,H,N,d] tensors, flattened, as the strided entry points take them."""
+    vals = []
+    for t in tensors:
+        vals += [t.stride(0), t.stride(1), t.stride(2)]
+    return (ctypes.c_int64 * len(vals))(*vals)

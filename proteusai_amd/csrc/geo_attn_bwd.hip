@@ -60,6 +60,9 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
 }
 
+// Element strides (batch, head, token) of Q, K, V, dO (bf16) and dQ, dK, dV (f32); the head dimension is contiguous.
+struct GbStrides { long q[3], k[3], v[3], g[3], dq[3], dk[3], dv[3]; };
+
 template <bool OWN_Q, bool LEGACY>
 __global__ __launch_bounds__(GB_THREADS, 2)
 void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
@@ -69,7 +72,7 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                          const float* __restrict__ Lse, const float* __restrict__ Dvec,
                          float* __restrict__ dQ, float* __restrict__ dK, float* __restrict__ dV,
                          float* __restrict__ d_sigma, float* __restrict__ d_beta,
-                         const int H, const int N, const int n_otiles, const float min_rbf, const float max_rbf)
+                         const int H, const int N, const int n_otiles, const float min_rbf, const float max_rbf, const GbStrides st)
 {
     __shared__ BwdSmem sm;
 
@@ -83,11 +86,12 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int zh = blockIdx.x / n_otiles;
     const int z  = zh / H;
     const int h  = zh - z * H;
-    const size_t head_off = (size_t)zh * (size_t)N * GB_D;
+    const size_t lin_off = (size_t)zh * (size_t)N;         // L and D are contiguous [Z,H,N]
+    auto at = [&](const long (&t)[3]) { return (size_t)z * (size_t)t[0] + (size_t)h * (size_t)t[1]; };
     const float*   cz = coords + (size_t)z * N * 3;
     const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
-    const float*   Lh = Lse + (size_t)zh * N;
-    const float*   Dh = Dvec + (size_t)zh * N;
+    const float*   Lh = Lse + lin_off;
+    const float*   Dh = Dvec + lin_off;
 
     const float sg  = sigma[h];
     const float cs2 = 0.72134752044448170368f / (sg * sg);       // log2(e)/2 / sigma^2: rbf = exp2(-d^2 cs2)
@@ -128,13 +132,14 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // exp2(-d^2 cs2) < 2^-25 beyond this distance: s*(1+rbf) rounds to s in fp32
     const float far2 = 25.0f / cs2;
     // B operands: lane (half, col) holds d = 16*ks + 8*half + 0..7 of its own token; the first one carries 1/sqrt(64)
-    const uint16_t* Bs_src = (OWN_Q ? Q : K) + head_off;
-    const uint16_t* Bp_src = (OWN_Q ? dO : V) + head_off;
+    const uint16_t* Bs_src = OWN_Q ? Q + at(st.q) : K + at(st.k);
+    const uint16_t* Bp_src = OWN_Q ? dO + at(st.g) : V + at(st.v);
+    const size_t bs_pitch = (size_t)(OWN_Q ? st.q[2] : st.k[2]), bp_pitch = (size_t)(OWN_Q ? st.g[2] : st.v[2]);
     bf16x8 bs[4], bp[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-        const uint4 r0 = *reinterpret_cast<const uint4*>(Bs_src + (size_t)oc * GB_D + ks * 16 + half * 8);
-        const uint4 r1 = *reinterpret_cast<const uint4*>(Bp_src + (size_t)oc * GB_D + ks * 16 + half * 8);
+        const uint4 r0 = *reinterpret_cast<const uint4*>(Bs_src + (size_t)oc * bs_pitch + ks * 16 + half * 8);
+        const uint4 r1 = *reinterpret_cast<const uint4*>(Bp_src + (size_t)oc * bp_pitch + ks * 16 + half * 8);
         bf16x8 v = __builtin_bit_cast(bf16x8, own_use ? r0 : make_uint4(0u, 0u, 0u, 0u));
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
@@ -156,8 +161,10 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // staging roles: a thread moves the 8-wide d chunk `dc` of the token pair `kp`
     const int kp = tid & 31;
     const int dc = tid >> 5;
-    const uint16_t* Ra_src = (OWN_Q ? K : Q) + head_off;
-    const uint16_t* Rb_src = (OWN_Q ? V : dO) + head_off;
+    const uint16_t* Ra_src = OWN_Q ? K + at(st.k) : Q + at(st.q);
+    const uint16_t* Rb_src = OWN_Q ? V + at(st.v) : dO + at(st.g);
+    // element offsets inside a (batch, head) slice fit 31 bits (checked on the host)
+    const int ra_pitch = (int)(OWN_Q ? st.k[2] : st.q[2]), rb_pitch = (int)(OWN_Q ? st.v[2] : st.g[2]);
 
     // registers holding the tile in flight from global memory: requested before the current tile is
     // computed, written to LDS after it (padded tokens as zeros)
@@ -170,10 +177,10 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     auto load_tile = [&](const int j0) {
         gj0 = j0;
         const int ta_ = min(j0 + 2 * kp, N - 1), tb_ = min(j0 + 2 * kp + 1, N - 1);
-        ga0 = *reinterpret_cast<const uint4*>(Ra_src + (size_t)ta_ * GB_D + dc * 8);
-        ga1 = *reinterpret_cast<const uint4*>(Ra_src + (size_t)tb_ * GB_D + dc * 8);
-        gb0 = *reinterpret_cast<const uint4*>(Rb_src + (size_t)ta_ * GB_D + dc * 8);
-        gb1 = *reinterpret_cast<const uint4*>(Rb_src + (size_t)tb_ * GB_D + dc * 8);
+        ga0 = *reinterpret_cast<const uint4*>(Ra_src + (ta_ * ra_pitch + dc * 8));
+        ga1 = *reinterpret_cast<const uint4*>(Ra_src + (tb_ * ra_pitch + dc * 8));
+        gb0 = *reinterpret_cast<const uint4*>(Rb_src + (ta_ * rb_pitch + dc * 8));
+        gb1 = *reinterpret_cast<const uint4*>(Rb_src + (tb_ * rb_pitch + dc * 8));
         if (mz) { gm0 = mz[ta_]; gm1 = mz[tb_]; }
         if (tid < GB_BN) {
             const int tc = min(j0 + tid, N - 1);
@@ -371,8 +378,8 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 
     // ---- epilogue: lane (half, col) holds d = dt*32 + 8*g + 4*half + 0..3 of its own token ----
     if (own_in) {
-        float* out_a = (OWN_Q ? dQ : dK) + head_off + (size_t)o * GB_D;
-        float* out_b = dV + head_off + (size_t)o * GB_D;
+        float* out_a = OWN_Q ? dQ + at(st.dq) + (size_t)o * (size_t)st.dq[2] : dK + at(st.dk) + (size_t)o * (size_t)st.dk[2];
+        float* out_b = dV + at(st.dv) + (size_t)o * (size_t)st.dv[2];
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -405,15 +412,39 @@ template <bool LEGACY>
 int launch_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
                const float* coords, const float* sigma, const float* beta, const uint8_t* mask,
                const float* L, const float* D, float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
-               int Z, int H, int N, float min_rbf, float max_rbf, hipStream_t st)
+               int Z, int H, int N, float min_rbf, float max_rbf, const GbStrides& gs, hipStream_t st)
 {
     const int n_otiles = (N + GB_OWN - 1) / GB_OWN;
     dim3 grid((unsigned)n_otiles * (unsigned)(Z * H), 1, 1);
     hipLaunchKernelGGL((geo_attn_bwd_kernel<false, LEGACY>), grid, dim3(GB_THREADS), 0, st,
-                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf);
+                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf, gs);
     hipLaunchKernelGGL((geo_attn_bwd_kernel<true, LEGACY>), grid, dim3(GB_THREADS), 0, st,
-                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf);
+                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf, gs);
     return (int)hipGetLastError();
+}
+
+GbStrides contiguous_strides(int H, int N) {
+    GbStrides gs;
+    const long t[3] = {(long)H * N * GB_D, (long)N * GB_D, (long)GB_D};
+    long* all[7] = {gs.q, gs.k, gs.v, gs.g, gs.dq, gs.dk, gs.dv};
+    for (int a = 0; a < 7; ++a) for (int i = 0; i < 3; ++i) all[a][i] = t[i];
+    return gs;
+}
+
+// strides[21]: (batch, head, token) element strides of Q, K, V, dO, dQ, dK, dV in this order
+int strides_from(const int64_t* strides, int Z, int H, int N, GbStrides& gs) {
+    if (!strides) return PROTEUS_ERR_NULL_POINTER;
+    long* dst[7] = {gs.q, gs.k, gs.v, gs.g, gs.dq, gs.dk, gs.dv};
+    for (int t = 0; t < 7; ++t) {
+        const int64_t sz = strides[3 * t], sh = strides[3 * t + 1], sn = strides[3 * t + 2];
+        if (sz < 0 || sh < 0 || sn < GB_D) return PROTEUS_ERR_BAD_LAYOUT;
+        const int align = (t >= 4) ? 4 : 8;            // 16-byte rows: f32 outputs, bf16 inputs
+        if ((sz % align) || (sh % align) || (sn % align)) return PROTEUS_ERR_BAD_ALIGNMENT;
+        if ((Z > 1 && sz == 0) || (H > 1 && sh == 0)) return PROTEUS_ERR_BAD_LAYOUT;
+        if ((long)N * sn >= (1L << 30)) return PROTEUS_ERR_BAD_SHAPE;
+        dst[t][0] = (long)sz; dst[t][1] = (long)sh; dst[t][2] = (long)sn;
+    }
+    return PROTEUS_OK;
 }
 
 }  // namespace
@@ -448,7 +479,43 @@ extern "C" int proteus_geo_attn_bwd(const uint16_t* Q, const uint16_t* K, const 
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (beta)
         return launch_bwd<true>(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV, d_sigma, d_beta,
-                                Z, H, N, min_rbf, max_rbf, st);
+                                Z, H, N, min_rbf, max_rbf, contiguous_strides(H, N), st);
     return launch_bwd<false>(Q, K, V, dO, coords, sigma, nullptr, key_pad_mask, L, D, dQ, dK, dV, d_sigma, nullptr,
-                             Z, H, N, 0.f, 1.f, st);
+                             Z, H, N, 0.f, 1.f, contiguous_strides(H, N), st);
+}
+
+extern "C" int proteus_geo_attn_bwd_strided_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                                  const int64_t* strides,
+                                                  const float* coords, const float* sigma, const float* beta,
+                                                  const uint8_t* key_pad_mask, const float* L, const float* D,
+                                                  const float* dQ, const float* dK, const float* dV,
+                                                  const float* d_sigma, const float* d_beta,
+                                                  int Z, int H, int N, int d_head, float min_rbf, float max_rbf)
+{
+    const int rc = proteus_geo_attn_bwd_check(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV,
+                                              d_sigma, d_beta, Z, H, N, d_head, min_rbf, max_rbf);
+    if (rc != PROTEUS_OK) return rc;
+    GbStrides gs;
+    return strides_from(strides, Z, H, N, gs);
+}
+
+extern "C" int proteus_geo_attn_bwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
+                                            const int64_t* strides,
+                                            const float* coords, const float* sigma, const float* beta,
+                                            const uint8_t* key_pad_mask, const float* L, const float* D,
+                                            float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
+                                            int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream)
+{
+    int rc = proteus_geo_attn_bwd_check(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV,
+                                        d_sigma, d_beta, Z, H, N, d_head, min_rbf, max_rbf);
+    if (rc != PROTEUS_OK) return rc;
+    GbStrides gs;
+    rc = strides_from(strides, Z, H, N, gs);
+    if (rc != PROTEUS_OK) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (beta)
+        return launch_bwd<true>(Q, K, V, dO, coords, sigma, beta, key_pad_mask, L, D, dQ, dK, dV, d_sigma, d_beta,
+                                Z, H, N, min_rbf, max_rbf, gs, st);
+    return launch_bwd<false>(Q, K, V, dO, coords, sigma, nullptr, key_pad_mask, L, D, dQ, dK, dV, d_sigma, nullptr,
+                             Z, H, N, 0.f, 1.f, gs, st);
 }

@@ -72,6 +72,9 @@ constexpr float GA_FAR = 5.0f;
 constexpr float GA_REBASE     = 20.0f;
 constexpr float GA_REBASE_SUM = 16777216.0f;
 
+// Element strides (batch, head, token) of Q, K, V (bf16) and O (f32); the head dimension is contiguous.
+struct GaStrides { long q[3], k[3], v[3], o[3]; };
+
 // One staged key tile.  Two of them are kept so that the next tile can be written
 // while the current one is still being read (one barrier per tile).
 struct __align__(16) TileBuf {
@@ -132,7 +135,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
                          const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                          float* __restrict__ O, float* __restrict__ L,
                          const int H, const int N, const int ZH, const int n_qtiles, const int take_all,
-                         const float* __restrict__ beta, const float min_rbf, const float max_rbf)
+                         const float* __restrict__ beta, const float min_rbf, const float max_rbf, const GaStrides st)
 {
     __shared__ Smem sm;
 
@@ -163,10 +166,12 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     }
     const int z  = zh / H;
     const int h  = zh - z * H;
-    const size_t head_off = (size_t)zh * (size_t)N * GA_D;
-    const uint16_t* Qh = Q + head_off;
-    const uint16_t* Kh = K + head_off;
-    const uint16_t* Vh = V + head_off;
+    const uint16_t* Qh = Q + (size_t)z * st.q[0] + (size_t)h * st.q[1];
+    const uint16_t* Kh = K + (size_t)z * st.k[0] + (size_t)h * st.k[1];
+    const uint16_t* Vh = V + (size_t)z * st.v[0] + (size_t)h * st.v[1];
+    float*          Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
+    const size_t q_pitch = (size_t)st.q[2], o_pitch = (size_t)st.o[2];
+    const int    k_pitch = (int)st.k[2] * 2, v_pitch = (int)st.v[2] * 2;      // bytes; N * pitch fits 31 bits (checked on the host)
     const float*    cz = coords + (size_t)z * N * 3;
     const uint8_t*  mz = key_pad ? key_pad + (size_t)z * N : nullptr;
 
@@ -209,7 +214,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
 #pragma unroll
             for (int b = 0; b < GA_QB; ++b) {
                 if (!q_in[b]) continue;
-                float* orow = O + head_off + (size_t)q[b] * GA_D;
+                float* orow = Oh + (size_t)q[b] * o_pitch;
 #pragma unroll
                 for (int g = 0; g < 8; ++g)
                     *reinterpret_cast<float4*>(orow + 8 * g + 4 * half) = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -280,7 +285,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         const int qc = q_ok[b] ? q[b] : q_mirror;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(Qh + (size_t)qc * GA_D + ks * 16 + half * 8);
+            const uint4 raw = *reinterpret_cast<const uint4*>(Qh + (size_t)qc * q_pitch + ks * 16 + half * 8);
             bf16x8 v = __builtin_bit_cast(bf16x8, raw);
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * 0.125f);
@@ -352,22 +357,22 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     unsigned mbyte = 0;                     // raw padding byte of key tid (threads < 64)
     unsigned mk0 = 0, mk1 = 0, mv0 = 0, mv1 = 0, mg = 0;   // raw padding bytes of the keys this thread stages
     int loaded_j0 = 0;
-    const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)Kh, 0, N * GA_D * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)Vh, 0, N * GA_D * 2, 0x00020000);
+    // the range ends with the last row, so rows past the end of the sequence read as zeros whatever lies behind them
+    const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)Kh, 0, (N - 1) * k_pitch + GA_D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)Vh, 0, (N - 1) * v_pitch + GA_D * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t rC = __builtin_amdgcn_make_buffer_rsrc((void*)cz, 0, N * 12, 0x00020000);
     const __amdgpu_buffer_rsrc_t rM = __builtin_amdgcn_make_buffer_rsrc((void*)(mz ? mz : key_pad), 0, mz ? N : 0, 0x00020000);
-    const int koff = (krow * GA_D + kdc * 8) * 2;            // byte offsets inside a tile
-    const int voff = (2 * kp * GA_D + vdc * 8) * 2;
+    const int koff = krow * k_pitch + kdc * 16;              // byte offsets inside a tile
+    const int voff = 2 * kp * v_pitch + vdc * 16;
     const int goff = 12 * gkey;
 
     auto load_tile = [&](const int j0) {
         loaded_j0 = j0;
         // the tile offset goes into the lane offset, not the scalar offset: only the former is range-checked
-        const int tile_bytes = j0 * GA_D * 2;
-        kreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + tile_bytes, 0, 0);
-        kreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + tile_bytes + 32 * GA_D * 2, 0, 0);
-        vreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + tile_bytes, 0, 0);
-        vreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + tile_bytes + GA_D * 2, 0, 0);
+        kreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + j0 * k_pitch, 0, 0);
+        kreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koff + (j0 + 32) * k_pitch, 0, 0);
+        vreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + j0 * v_pitch, 0, 0);
+        vreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rV, voff + (j0 + 1) * v_pitch, 0, 0);
         graw    = __builtin_amdgcn_raw_buffer_load_b128(rC, goff + j0 * 12, 0, 0);
         if (mz) {
             mbyte = __builtin_amdgcn_raw_buffer_load_b8(rM, lane + j0, 0, 0);      // used by wave 0 only
@@ -637,7 +642,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
         const bool  row_ok = q_ok[b] && l_tot > 0.f;
         const float inv_l = row_ok ? 1.0f / l_tot : 0.f;
         if (q_in[b]) {
-            float* orow = O + head_off + (size_t)q[b] * GA_D;
+            float* orow = Oh + (size_t)q[b] * o_pitch;
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -684,7 +689,7 @@ namespace {
 template <bool LEGACY, int QB>
 int launch_attn_qb(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                    const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int dist,
-                   const float* beta, float min_rbf, float max_rbf, hipStream_t st)
+                   const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
 {
     constexpr int BM = GA_WAVES * 32 * QB;
     const int n_qtiles = (N + BM - 1) / BM;
@@ -694,17 +699,17 @@ int launch_attn_qb(const uint16_t* Q, const uint16_t* K, const uint16_t* V, cons
     // 1 / 2: force the matrix-core / vector-ALU path everywhere
     if (dist != 2)
         hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 1 ? 1 : 0, beta, min_rbf, max_rbf);
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 1 ? 1 : 0, beta, min_rbf, max_rbf, gs);
     if (dist != 1)
         hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 2 ? 1 : 0, beta, min_rbf, max_rbf);
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 2 ? 1 : 0, beta, min_rbf, max_rbf, gs);
     return (int)hipGetLastError();
 }
 
 template <bool LEGACY>
 int launch_attn(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                 const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
-                const float* beta, float min_rbf, float max_rbf, hipStream_t st)
+                const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
 {
     // Two query blocks per wave unless that leaves at most one workgroup per compute unit (256 of them on
     // this chip, two workgroups each): then one block per wave doubles the waves in flight.
@@ -713,10 +718,62 @@ int launch_attn(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const f
     int dist = tuning;
     if (tuning == 3) { one_block = true;  dist = 0; }
     if (tuning == 4) { one_block = false; dist = 0; }
-    return one_block ? launch_attn_qb<LEGACY, 1>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, st)
-                     : launch_attn_qb<LEGACY, 2>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, st);
+    return one_block ? launch_attn_qb<LEGACY, 1>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, gs, st)
+                     : launch_attn_qb<LEGACY, 2>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, gs, st);
+}
+// contiguous [Z,H,N,64] tensors
+GaStrides contiguous_strides(int H, int N) {
+    GaStrides gs;
+    const long t[3] = {(long)H * N * GA_D, (long)N * GA_D, (long)GA_D};
+    for (int i = 0; i < 3; ++i) { gs.q[i] = t[i]; gs.k[i] = t[i]; gs.v[i] = t[i]; gs.o[i] = t[i]; }
+    return gs;
+}
+
+// strides[12]: (batch, head, token) element strides of Q, K, V, O in this order
+int strides_from(const int64_t* strides, int Z, int H, int N, GaStrides& gs) {
+    if (!strides) return PROTEUS_ERR_NULL_POINTER;
+    long* dst[4] = {gs.q, gs.k, gs.v, gs.o};
+    for (int t = 0; t < 4; ++t) {
+        const int64_t sz = strides[3 * t], sh = strides[3 * t + 1], sn = strides[3 * t + 2];
+        // rows of 64 contiguous elements that do not overlap and stay 16-byte aligned; a sequence's byte
+        // offsets fit the 31 bits of a buffer-load offset
+        if (sz < 0 || sh < 0 || sn < GA_D) return PROTEUS_ERR_BAD_LAYOUT;
+        const int align = (t == 3) ? 4 : 8;
+        if ((sz % align) || (sh % align) || (sn % align)) return PROTEUS_ERR_BAD_ALIGNMENT;
+        if ((Z > 1 && sz == 0) || (H > 1 && sh == 0)) return PROTEUS_ERR_BAD_LAYOUT;
+        if ((long)N * sn * (t == 3 ? 4 : 2) >= (1L << 31)) return PROTEUS_ERR_BAD_SHAPE;
+        dst[t][0] = (long)sz; dst[t][1] = (long)sh; dst[t][2] = (long)sn;
+    }
+    return PROTEUS_OK;
 }
 }  // namespace
+
+extern "C" int proteus_geo_attn_fwd_strided_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                                  const int64_t* strides,
+                                                  const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                                  const float* O, const float* L,
+                                                  int Z, int H, int N, int d_head, int tuning)
+{
+    const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    GaStrides gs;
+    return strides_from(strides, Z, H, N, gs);
+}
+
+extern "C" int proteus_geo_attn_fwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                            const int64_t* strides,
+                                            const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                            float* O, float* L,
+                                            int Z, int H, int N, int d_head, int tuning, void* stream)
+{
+    int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    GaStrides gs;
+    rc = strides_from(strides, Z, H, N, gs);
+    if (rc != PROTEUS_OK) return rc;
+    return launch_attn<false>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f, gs,
+                              reinterpret_cast<hipStream_t>(stream));
+}
 
 extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                                     const float* coords, const float* sigma,
@@ -726,7 +783,7 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
 {
     const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
     if (rc != PROTEUS_OK) return rc;
-    return launch_attn<false>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f,
+    return launch_attn<false>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f, contiguous_strides(H, N),
                               reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -743,6 +800,6 @@ extern "C" int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K,
     if (!(max_rbf > min_rbf)) return PROTEUS_ERR_BAD_SHAPE;
     // a pair mask makes the result sensitive to the last bits of the rbf: use direct distances then
     if ((tuning == 0 || tuning >= 3) && (min_rbf > 0.f || max_rbf < 1.f)) tuning = 2;
-    return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf,
+    return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf, contiguous_strides(H, N),
                              reinterpret_cast<hipStream_t>(stream));
 }

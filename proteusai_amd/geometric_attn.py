@@ -12,8 +12,32 @@ import torch.nn as nn
 from . import _lib
 
 
+def _rows_ok(t, itemsize):
+    """Can the kernels read / write this [Z,H,N,d] tensor in place?  Rows of d contiguous elements, 16-byte
+    aligned, no negative or overlapping-row strides; the batch, head and token strides are otherwise free."""
+    per16 = 16 // itemsize
+    return (t.stride(3) == 1 and t.data_ptr() % 16 == 0 and t.stride(2) >= t.size(3)
+            and all(st >= 0 and st % per16 == 0 for st in t.stride()[:3])
+            and (t.size(0) == 1 or t.stride(0) > 0) and (t.size(1) == 1 or t.stride(1) > 0)
+            and t.size(2) * t.stride(2) * itemsize < 2 ** 31)
+
+
+def _operand(t):
+    """bf16 view of an operand the kernels can read where it lies (a copy only if it has to be cast or its rows
+    are not contiguous)."""
+    t = t.detach()
+    if t.dtype != torch.bfloat16:
+        t = t.to(torch.bfloat16)
+    return t if _rows_ok(t, 2) else t.contiguous()
+
+
+def _is_plain(*ts):
+    return all(t.is_contiguous() for t in ts)
+
+
 def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0,
-             betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0, check_sigma: bool = True):
+             betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0, check_sigma: bool = True,
+             token_major_out: bool = False):
     """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None).
 
     Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569),
@@ -21,6 +45,11 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     key_padding_mask: True = padded.  Padded query rows and rows without a
     valid key give O = 0 and logsumexp = -inf.  With return_lse the
     logsumexp L [Z,H,N] is returned as well.
+
+    Q, K, V may be views with any batch / head / token strides as long as the rows of d elements are
+    contiguous and 16-byte aligned (e.g. slices of a fused [Z,N,3,H,d] projection): they are read in place.
+    token_major_out=True returns O as a [Z,H,N,d] view of memory laid out [Z,N,H,d] (what a following
+    projection over the concatenated heads reads without a copy).
 
     With `betas` [H] the logits are those of the reference's kernel instead,
     S + beta_h*(2(rbf-min_rbf)/(max_rbf-min_rbf)-1)*|S| with pairs whose rbf lies outside
@@ -42,9 +71,11 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         raise AssertionError(f"spreads must be a tensor of positive, non-zero floats, not {sigma}")
     lib = _lib.load()
     dev = Q.device
-    q = Q.detach().to(torch.bfloat16).contiguous()
-    k = K.detach().to(torch.bfloat16).contiguous()
-    v = V.detach().to(torch.bfloat16).contiguous()
+    legacy = betas is not None
+    if legacy:      # the beta-weighted logits have no strided entry point
+        q, k, v = (t.detach().to(torch.bfloat16).contiguous() for t in (Q, K, V))
+    else:
+        q, k, v = _operand(Q), _operand(K), _operand(V)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
     m = None
@@ -52,16 +83,23 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         if tuple(key_padding_mask.shape) != (Z, N):
             raise AssertionError(f"mask must be of shape ({Z}, {N}), not {tuple(key_padding_mask.shape)}")
         m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
-    O = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
+    if token_major_out and not legacy:
+        O = torch.empty(Z, N, H, d, dtype=torch.float32, device=dev).permute(0, 2, 1, 3)
+    else:
+        O = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
     L = torch.empty(Z, H, N, dtype=torch.float32, device=dev)
     if Z == 0 or H == 0 or N == 0:
         return (O, L) if return_lse else O
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        if betas is None:
+        if not legacy and _is_plain(q, k, v, O):
             rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
                                           None if m is None else m.data_ptr(),
                                           O.data_ptr(), L.data_ptr(), Z, H, N, d, int(tuning), stream)
+        elif not legacy:
+            rc = lib.proteus_geo_attn_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.stride_array(q, k, v, O),
+                                                  c.data_ptr(), s.data_ptr(), None if m is None else m.data_ptr(),
+                                                  O.data_ptr(), L.data_ptr(), Z, H, N, d, int(tuning), stream)
         else:
             if betas.dim() != 1 or betas.size(0) != H:
                 raise AssertionError(f"number of betas must be equal to nheads, not {tuple(betas.shape)} and {H=}")
@@ -86,11 +124,9 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
         raise _lib.ProteusError("geo_attn_backward needs tensors on the GPU (there is no CPU path)")
     lib = _lib.load()
     dev = Q.device
-    q = Q.detach().to(torch.bfloat16).contiguous()
-    k = K.detach().to(torch.bfloat16).contiguous()
-    v = V.detach().to(torch.bfloat16).contiguous()
+    q, k, v = _operand(Q), _operand(K), _operand(V)
     D = torch.sum(O.detach().float() * dO.detach().float(), dim=3).contiguous()
-    do = dO.detach().to(torch.bfloat16).contiguous()
+    do = _operand(dO)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
     lse = L.detach().to(torch.float32).contiguous()
@@ -98,20 +134,26 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     if key_padding_mask is not None:
         m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
     bt = None if betas is None else betas.detach().to(device=dev, dtype=torch.float32).contiguous()
-    dQ = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
-    dK = torch.empty_like(dQ)
-    dV = torch.empty_like(dQ)
+    # gradients in the memory order of their operands (dense), so that what consumes them needs no reshuffle
+    def like(t):
+        g = torch.empty_like(t, dtype=torch.float32)
+        return g if _rows_ok(g, 4) else torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
+    dQ, dK, dV = like(Q), like(K), like(V)
     d_sigma = torch.zeros(H, dtype=torch.float32, device=dev)
     d_beta = None if bt is None else torch.zeros(H, dtype=torch.float32, device=dev)
     if Z == 0 or H == 0 or N == 0:
         return dQ, dK, dV, d_sigma, d_beta
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), c.data_ptr(), s.data_ptr(),
-                                      None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
-                                      lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
-                                      d_sigma.data_ptr(), None if d_beta is None else d_beta.data_ptr(),
-                                      Z, H, N, d, float(min_rbf), float(max_rbf), stream)
+        tail = (c.data_ptr(), s.data_ptr(), None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
+                lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
+                d_sigma.data_ptr(), None if d_beta is None else d_beta.data_ptr(),
+                Z, H, N, d, float(min_rbf), float(max_rbf), stream)
+        if _is_plain(q, k, v, do, dQ, dK, dV):
+            rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), *tail)
+        else:
+            rc = lib.proteus_geo_attn_bwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(),
+                                                  _lib.stride_array(q, k, v, do, dQ, dK, dV), *tail)
     _lib.check(rc, "proteus_geo_attn_bwd")
     return dQ, dK, dV, d_sigma, d_beta
 
@@ -121,12 +163,14 @@ class _geometric_attn(torch.autograd.Function):
     flows to the coordinates, as in the reference."""
 
     @staticmethod
-    def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf, check_sigma=True):
+    def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf, check_sigma=True,
+                token_major_out=False, out_dtype=None):
         O, L = geo_attn(Q, K, V, coords, spreads, key_padding_mask, return_lse=True, betas=betas,
-                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma)
+                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma, token_major_out=token_major_out)
         ctx.save_for_backward(Q, K, V, O, L, coords, spreads, betas, key_padding_mask)
         ctx.min_rbf, ctx.max_rbf = min_rbf, max_rbf
-        return O
+        # the fp32 O is what the backward reads; the caller may ask for it in its own working precision
+        return O if out_dtype is None or out_dtype == O.dtype else O.to(out_dtype)
 
     @staticmethod
     def backward(ctx, dO):
@@ -134,19 +178,24 @@ class _geometric_attn(torch.autograd.Function):
         dQ, dK, dV, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
                                                         ctx.min_rbf, ctx.max_rbf)
         return (dQ.to(Q.dtype), dK.to(K.dtype), dV.to(V.dtype), None, d_sigma.to(spreads.dtype),
-                None if betas is None else d_beta.to(betas.dtype), None, None, None, None)
+                None if betas is None else d_beta.to(betas.dtype), None, None, None, None, None, None)
 
 
-def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True):
+def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True,
+                   token_major_out=False, out_dtype=None):
     """Same call as the reference's geometric_attn (geometric_attn.py:545-548).
 
     betas=None selects the README logits S*(1+RBF) (README.md:40; the rbf range must then be the full
     [0, 1]); a betas tensor selects the reference kernel's own logits S + beta*RBF_norm*|S| with its
     [min_rbf, max_rbf] pair mask (geometric_attn.py:193-201).
+
+    Beyond the reference's call: token_major_out lays O out [Z,N,H,d] in memory (returned as a [Z,H,N,d] view),
+    out_dtype returns O in another dtype than fp32 (the fp32 result is kept for the backward either way).
     """
     if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
         raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
-    return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads)
+    return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads,
+                                 token_major_out, out_dtype)
 
 
 class GeoAttention(nn.Module):
@@ -193,31 +242,48 @@ class GeoAttention(nn.Module):
         batch, N, d_model = q.shape
         assert d_model == self.d_model
         # Per-head projections x @ W_h + b_h (encoder.py:99-101) as plain GEMMs against the heads' weights laid
-        # side by side, [d_model, heads*d_k]: the broadcast batched matmul of the reference materialises the
-        # activations once per head.  Self-attention takes one GEMM for all three.
+        # side by side, [d_model, heads*d_k] (the broadcast batched matmul of the reference materialises the
+        # activations once per head); self-attention takes one GEMM for all three.  The kernels read Q, K, V
+        # where the GEMM left them ([Z,N,(3,)H,d_k], as strided [Z,H,N,d_k] views) and write O token-major, so
+        # no head split or merge is ever copied.
         H, dk = self.heads, self.d_k
 
-        def flat(w):                       # [H, d_model, d_k] -> [d_model, H*d_k]
-            return w.permute(1, 0, 2).reshape(self.d_model, H * dk)
-
-        def heads_first(x):                # [Z, N, H*d_k] -> [Z, H, N, d_k]
+        def heads_first(x):                # [Z, N, H*d_k] -> [Z, H, N, d_k] view
             return x.view(batch, N, H, dk).permute(0, 2, 1, 3)
         if q is k and k is v:
-            w = torch.cat([flat(self.q_proj), flat(self.k_proj), flat(self.v_proj)], dim=1)
-            b = torch.cat([self.q_bias.reshape(-1), self.k_bias.reshape(-1), self.v_bias.reshape(-1)])
+            w, b = self._fused_qkv()
             qkv = torch.addmm(b, q.reshape(batch * N, d_model), w).view(batch, N, 3, H * dk)
             Q, K, V = heads_first(qkv[:, :, 0]), heads_first(qkv[:, :, 1]), heads_first(qkv[:, :, 2])
         else:
+            def flat(w_):                  # [H, d_model, d_k] -> [d_model, H*d_k]
+                return w_.permute(1, 0, 2).reshape(self.d_model, H * dk)
             Q = heads_first(torch.addmm(self.q_bias.reshape(-1), q.reshape(batch * N, d_model), flat(self.q_proj)))
             K = heads_first(torch.addmm(self.k_bias.reshape(-1), k.reshape(batch * N, d_model), flat(self.k_proj)))
             V = heads_first(torch.addmm(self.v_bias.reshape(-1), v.reshape(batch * N, d_model), flat(self.v_proj)))
         # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
         if self.legacy_logits:
             out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf,
-                                 max_rbf=self.max_rbf, check_spreads=False)
+                                 max_rbf=self.max_rbf, check_spreads=False, out_dtype=q.dtype)
         else:
-            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False)
-        out = out.to(q.dtype)
-        out = out.permute(0, 2, 3, 1)                    # batch x N x d_k x heads
-        out = out.reshape(batch, N, self.d_model)
-        return self.out_proj(out)
+            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False,
+                                 token_major_out=True, out_dtype=q.dtype)
+        # The reference concatenates the heads as a (d_k x heads) interleave (encoder.py:114-115) before the output
+        # projection.  Token-major O is the (heads x d_k) order; the same product is taken against the projection's
+        # input columns in that order instead of reshuffling the activations.
+        out = out.permute(0, 2, 1, 3).reshape(batch, N, self.d_model)           # a view when O is token-major
+        w_o = self.out_proj.weight.view(self.d_model, dk, H).permute(0, 2, 1).reshape(self.d_model, self.d_model)
+        return torch.nn.functional.linear(out, w_o)
+
+    def _fused_qkv(self):
+        """[d_model, 3*H*d_k] weight and [3*H*d_k] bias of the fused self-attention projection.  Rebuilt from the
+        per-head parameters whenever they may have changed; kept across calls only where no gradient is needed."""
+        params = (self.q_proj, self.k_proj, self.v_proj, self.q_bias, self.k_bias, self.v_bias)
+        keep = not (torch.is_grad_enabled() and any(p.requires_grad for p in params))
+        key = tuple((p._version, p.data_ptr(), p.dtype) for p in params)
+        if keep and getattr(self, "_qkv_cache", None) is not None and self._qkv_cache[0] == key:
+            return self._qkv_cache[1], self._qkv_cache[2]
+        H, dk = self.heads, self.d_k
+        w = torch.stack((self.q_proj, self.k_proj, self.v_proj)).permute(2, 0, 1, 3).reshape(self.d_model, 3 * H * dk)
+        b = torch.stack((self.q_bias, self.k_bias, self.v_bias)).reshape(-1)
+        self._qkv_cache = (key, w.detach(), b.detach()) if keep else None
+        return w, b

@@ -261,3 +261,38 @@ def test_we_backward_argument_validation_happens_before_any_hip_call():
     assert lib.proteus_we_aniso_bwd_check(p, None, None, None, None, p, need, 2, 100, 16) == -1
     assert lib.proteus_we_aniso_bwd_check(p, p, p, p, p, p, need - 4, 2, 100, 16) == -2
     assert lib.proteus_we_aniso_bwd(p, p, p, p, p, None, need, 2, 100, 16, None) == -1
+
+
+def test_strided_attention_argument_validation():
+    import ctypes
+    lib = _lib.load()
+    p = 0x1000
+    Z, H, N = 2, 4, 100
+
+    def arr(*v):
+        return (ctypes.c_int64 * len(v))(*v)
+    plain = [H * N * 64, N * 64, 64]
+    fused = [N * 3 * H * 64, 64, 3 * H * 64]                    # slices of [Z,N,3,H,d]
+    tok = [N * H * 64, 64, H * 64]                             # [Z,N,H,d]
+
+    def fwd(st):
+        return lib.proteus_geo_attn_fwd_strided_check(p, p, p, st, p, p, None, p, p, Z, H, N, 64, 0)
+    assert fwd(arr(*(plain * 4))) == 0
+    assert fwd(arr(*(fused * 3 + tok))) == 0
+    assert fwd(None) == -1
+    assert fwd(arr(*(plain * 3 + [H * N * 64, N * 64, 32]))) == -4       # rows would overlap
+    assert fwd(arr(*([-1, N * 64, 64] + plain * 3))) == -4
+    assert fwd(arr(*([0, N * 64, 64] + plain * 3))) == -4                # batch items on top of each other
+    assert fwd(arr(*([H * N * 64, N * 64, 68] + plain * 3))) == -5       # bf16 rows off 16-byte alignment
+    assert fwd(arr(*(plain * 3 + [H * N * 64, N * 64, 66]))) == -5       # f32 rows off 16-byte alignment
+    assert fwd(arr(*([H * N * 64, N * 64, 1 << 29] + plain * 3))) == -2  # offsets beyond 31 bits
+    assert lib.proteus_geo_attn_fwd_strided(None, p, p, arr(*(plain * 4)), p, p, None, p, p, Z, H, N, 64, 0, None) == -1
+
+    def bwd(st):
+        return lib.proteus_geo_attn_bwd_strided_check(p, p, p, p, st, p, p, None, None, p, p, p, p, p, p, None,
+                                                      Z, H, N, 64, 0.0, 1.0)
+    assert bwd(arr(*(plain * 7))) == 0
+    assert bwd(arr(*(fused * 3 + tok * 4))) == 0
+    assert bwd(None) == -1
+    assert bwd(arr(*(plain * 6 + [H * N * 64, N * 64, 63]))) == -4
+    assert bwd(arr(*(plain * 6 + [H * N * 64, N * 64, 66]))) == -5

@@ -151,3 +151,26 @@ def test_module_trains(gpu):
             continue
         assert p.grad is not None and torch.isfinite(p.grad).all(), name
     assert m.spread_weights.grad.abs().sum() > 0 and m.q_proj.grad.abs().sum() > 0
+
+
+def test_strided_operands_give_the_same_gradients(gpu):
+    """Operands as slices of a fused [Z,N,3,H,d] buffer, dO token-major: the strided entry point gives the
+    bits of the contiguous one (the per-head scalars are atomic sums: compared to rounding)."""
+    Z, H, N = 2, 2, 200
+    Q, K, V, dO, coords, sigma, mask = make(41, Z, H, N, maskfrac=0.1)
+    dev = lambda t: None if t is None else t.to(gpu)
+    O, L = pa.geo_attn(dev(Q), dev(K), dev(V), dev(coords), dev(sigma), dev(mask), return_lse=True)
+    ref = pa.geo_attn_backward(dev(Q), dev(K), dev(V), O, L, dev(dO).bfloat16(), dev(coords), dev(sigma), dev(mask))
+    fused = torch.stack([t.permute(0, 2, 1, 3) for t in (Q, K, V)], dim=2).contiguous().to(gpu)
+    Qs, Ks, Vs = (fused[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    dOs = dev(dO).bfloat16().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    Os = O.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    got = pa.geo_attn_backward(Qs, Ks, Vs, Os, L, dOs, dev(coords), dev(sigma), dev(mask))
+    torch.cuda.synchronize()
+    for name, x, y in zip(("dQ", "dK", "dV"), got[:3], ref[:3]):
+        assert torch.equal(x, y), name
+    assert torch.allclose(got[3], ref[3], rtol=1e-4, atol=1e-6)
+    # a dense head-major operand gets its gradient in the same memory order
+    Qh = dev(Q).permute(1, 0, 2, 3).contiguous().permute(1, 0, 2, 3)
+    got2 = pa.geo_attn_backward(Qh, dev(K), dev(V), O, L, dev(dO).bfloat16(), dev(coords), dev(sigma), dev(mask))
+    assert got2[0].stride() == Qh.stride() and torch.equal(got2[0], ref[0])

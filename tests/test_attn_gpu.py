@@ -143,6 +143,32 @@ def test_every_variant_matches_the_oracle(gpu):
         check((O.cpu().numpy(), L.cpu().numpy()), *a, what=f"variant {name}")
 
 
+def test_strided_operands_and_token_major_output_are_read_and_written_in_place(gpu):
+    """Q, K, V as slices of one fused [Z,N,3,H,d] buffer (what a fused projection leaves) and O laid out
+    [Z,N,H,d]: the same bits as from contiguous [Z,H,N,d] tensors, and nothing written outside O's rows."""
+    Z, H, N = 2, 3, 333
+    a = make(31, Z, H, N, maskfrac=0.1, tail=True)
+    Q, K, V, coords, sigma, mask = a
+    fused = torch.stack([t.permute(0, 2, 1, 3) for t in (Q, K, V)], dim=2).contiguous().to(gpu)      # [Z,N,3,H,d]
+    Qs, Ks, Vs = (fused[:, :, i].permute(0, 2, 1, 3) for i in range(3))                            # [Z,H,N,d] views
+    assert not Qs.is_contiguous() and Qs.stride(2) == 3 * H * 64
+    ref_O, ref_L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), return_lse=True)
+    O, L = pa.geo_attn(Qs, Ks, Vs, coords.to(gpu), sigma.to(gpu), mask.to(gpu), return_lse=True, token_major_out=True)
+    torch.cuda.synchronize()
+    assert O.shape == (Z, H, N, 64) and O.permute(0, 2, 1, 3).is_contiguous()
+    assert torch.equal(O, ref_O) and torch.equal(L, ref_L)
+    check((O.cpu().numpy(), L.cpu().numpy()), *a, what="strided")
+    # head-major batch order [H,Z,N,d] (what a per-head batched projection leaves)
+    Qh, Kh, Vh = (t.to(gpu).permute(1, 0, 2, 3).contiguous().permute(1, 0, 2, 3) for t in (Q, K, V))
+    O2 = pa.geo_attn(Qh, Kh, Vh, coords.to(gpu), sigma.to(gpu), mask.to(gpu))
+    assert torch.equal(O2, ref_O)
+    # rows that are not 16-byte aligned cannot be read in place: the wrapper copies, the result is the same
+    pad = torch.zeros(Z, H, N, 68, dtype=torch.bfloat16, device=gpu)
+    pad[..., 4:] = Q.to(gpu)
+    O3 = pa.geo_attn(pad[..., 4:], K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu))
+    assert torch.equal(O3, ref_O)
+
+
 def test_flat_multiplier_equals_sdpa_on_gpu(gpu):
     # sigma -> infinity: multiplier == 2 -> torch SDPA with scale 2/sqrt(d), evaluated in fp32 on the same bf16 values
     Q, K, V, coords, _, _ = make(3, 2, 4, 777)
