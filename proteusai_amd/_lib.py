@@ -137,3 +137,22 @@ def stride_array(*tensors):
     for t in tensors:
         vals += [t.stride(0), t.stride(1), t.stride(2)]
     return (ctypes.c_int64 * len(vals))(*vals)
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(dev):
+    """Context that makes `dev` the current device for the launch; free when it already is."""
+    import torch
+    if dev.index is None or torch.cuda.current_device() == dev.index:
+        return _NO_SWITCH
+    return torch.cuda.device(dev)

@@ -15,6 +15,8 @@ from . import _lib
 def _rows_ok(t, itemsize):
     """Can the kernels read / write this [Z,H,N,d] tensor in place?  Rows of d contiguous elements, 16-byte
     aligned, no negative or overlapping-row strides; the batch, head and token strides are otherwise free."""
+    if t.is_contiguous():
+        return t.data_ptr() % 16 == 0
     per16 = 16 // itemsize
     return (t.stride(3) == 1 and t.data_ptr() % 16 == 0 and t.stride(2) >= t.size(3)
             and all(st >= 0 and st % per16 == 0 for st in t.stride()[:3])
@@ -90,7 +92,7 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     L = torch.empty(Z, H, N, dtype=torch.float32, device=dev)
     if Z == 0 or H == 0 or N == 0:
         return (O, L) if return_lse else O
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         if not legacy and _is_plain(q, k, v, O):
             rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
@@ -125,7 +127,7 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     lib = _lib.load()
     dev = Q.device
     q, k, v = _operand(Q), _operand(K), _operand(V)
-    D = torch.sum(O.detach().float() * dO.detach().float(), dim=3).contiguous()
+    D = torch.sum(O.detach().float() * dO.detach(), dim=3).contiguous()       # fp32 by type promotion
     do = _operand(dO)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
@@ -143,7 +145,7 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     d_beta = None if bt is None else torch.zeros(H, dtype=torch.float32, device=dev)
     if Z == 0 or H == 0 or N == 0:
         return dQ, dK, dV, d_sigma, d_beta
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         tail = (c.data_ptr(), s.data_ptr(), None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
                 lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),

@@ -50,7 +50,7 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
     sin_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev) if need_sums else None
     if Z == 0 or N == 0 or K == 0:
         return out, cos_sums, sin_sums
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         if magnitude_type == 1:
             rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
@@ -84,7 +84,7 @@ def we_backward(dO, cos_sums, sin_sums):
     dk = torch.empty(K, dtype=torch.float32, device=dO.device)
     if Z == 0 or N == 0 or K == 0:
         return dk.zero_()
-    with torch.cuda.device(dO.device):
+    with _lib.on_device(dO.device):
         rc = lib.proteus_we_bwd(g.data_ptr(), c.data_ptr(), s.data_ptr(), dk.data_ptr(), ws.data_ptr(), ws.numel() * 4,
                                 Z, N, K, stream)
     _lib.check(rc, "proteus_we_bwd")
@@ -103,7 +103,7 @@ def we_aniso_backward(dO, d_cb=None, d_k=None):
     if Z == 0 or N == 0 or K == 0:
         return (None if g_cb is None else g_cb.zero_()), (None if g_k is None else g_k.zero_())
     ptr = lambda t: None if t is None else t.data_ptr()
-    with torch.cuda.device(dO.device):
+    with _lib.on_device(dO.device):
         rc = lib.proteus_we_aniso_bwd(g.data_ptr(), ptr(a), ptr(b), ptr(g_cb), ptr(g_k), ws.data_ptr(), ws.numel() * 4,
                                       Z, N, K, stream)
     _lib.check(rc, "proteus_we_aniso_bwd")
@@ -177,7 +177,7 @@ def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tu
     d_k = torch.empty_like(out)
     if Z == 0 or N == 0 or K == 0:
         return out, d_cb, d_k
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         rc = lib.proteus_we_aniso_fwd(a.data_ptr(), b.data_ptr(), _lib.COORDS_AOS, cb.data_ptr(), w.data_ptr(),
                                       None if m is None else m.data_ptr(),
