@@ -68,11 +68,23 @@ def test_attention_forward_and_backward(gpu, case):
     lo, hi = (0.02, 0.95) if legacy and case % 2 == 0 else (0.0, 1.0)
     what = f"case {case}: Z={Z} H={H} N={N} legacy={legacy}"
 
-    q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
     s = sigma.to(gpu).requires_grad_(True)
     bt = None if betas is None else betas.to(gpu).requires_grad_(True)
-    O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi)
-    O.backward(dO.to(gpu).float())
+    strided = (not legacy) and case % 2 == 1
+    what += f" strided={strided}"
+    if strided:
+        # operands as slices of one fused [Z,N,3,H,d] buffer, O token-major: read and written in place
+        fused = torch.stack([t.permute(0, 2, 1, 3) for t in (Q, K, V)], dim=2).contiguous().to(gpu).requires_grad_(True)
+        q, k, v = (fused[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi, token_major_out=True)
+        assert O.permute(0, 2, 1, 3).is_contiguous()
+        O.backward(dO.to(gpu).float())
+        gq, gk, gv = (fused.grad[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    else:
+        q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
+        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi)
+        O.backward(dO.to(gpu).float())
+        gq, gk, gv = q.grad, k.grad, v.grad
 
     rq, rk, rv = (t.double().requires_grad_(True) for t in (Q, K, V))
     rs = sigma.double().requires_grad_(True)
@@ -84,7 +96,7 @@ def test_attention_forward_and_backward(gpu, case):
     assert torch.isfinite(Og).all(), what
     assert (Og - Oref.detach()).abs().max() <= 2e-2, f"{what}: O {(Og - Oref.detach()).abs().max():.3e}"
     assert (Og[mask[:, None, :].expand(-1, H, -1)] == 0).all(), what
-    pairs = [(q.grad, rq.grad, "dQ"), (k.grad, rk.grad, "dK"), (v.grad, rv.grad, "dV"), (s.grad, rs.grad, "d_sigma")]
+    pairs = [(gq, rq.grad, "dQ"), (gk, rk.grad, "dK"), (gv, rv.grad, "dV"), (s.grad, rs.grad, "d_sigma")]
     if legacy:
         pairs.append((bt.grad, rb.grad, "d_beta"))
     for gg, rr, name in pairs:
