@@ -122,22 +122,23 @@ __device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
 }
 
 // DIST_VALU selects how the distances are evaluated: false = on the matrix cores, true = directly on
-// the vector ALU.  Both instantiations are launched over the same grid; unless take_all is set, a
-// workgroup runs in the matrix-core kernel if its queries lie within GA_MFMA_DIST_MAX_RHO2 of their
-// origin and in the vector-ALU kernel otherwise, and returns at once from the other one.
+// the vector ALU.  Unless take_all is set both bodies are run for every group of queries (by two
+// workgroups of one launch): a group is computed with the matrix-core distances if its queries lie
+// within GA_MFMA_DIST_MAX_RHO2 of their origin and with the direct ones otherwise, and the body that
+// does not own it returns after the prologue.
 // LEGACY selects the logits of the reference's Triton kernel instead of the README multiplier:
 //   s = S + beta_h * (2 (rbf - min_rbf)/(max_rbf - min_rbf) - 1) * |S|, pairs with rbf outside [min_rbf, max_rbf] masked
 //   (old/old_scripts/attn/geometric_attn.py:193-201).
 template <bool DIST_VALU, bool LEGACY, int GA_QB>
-__global__ __launch_bounds__(GA_THREADS, 2)
-void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
-                         const uint16_t* __restrict__ V, const float* __restrict__ coords,
-                         const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
-                         float* __restrict__ O, float* __restrict__ L,
-                         const int H, const int N, const int ZH, const int n_qtiles, const int take_all,
-                         const float* __restrict__ beta, const float min_rbf, const float max_rbf, const GaStrides st)
+__device__ __forceinline__
+void geo_attn_fwd_body(Smem& sm, const int block_id,
+                       const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                       const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                       const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                       float* __restrict__ O, float* __restrict__ L,
+                       const int H, const int N, const int ZH, const int n_qtiles, const int take_all,
+                       const float* __restrict__ beta, const float min_rbf, const float max_rbf, const GaStrides& st)
 {
-    __shared__ Smem sm;
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -152,7 +153,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     // paired with one for which it matters for few, so the XCDs finish together.
     int zh, qt;
     {
-        const int id = blockIdx.x;
+        const int id = block_id;
         if ((ZH & 7) == 0) {
             const int per_xcd = ZH >> 3;
             const int r = id >> 3;
@@ -210,7 +211,7 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int q_first = sm.q_first, q_last = sm.q_last;
     if (q_last < 0) {
         // every query of this workgroup is padded (or out of range): zeros, L = -inf, done
-        if (take_all || DIST_VALU) {      // exactly one of the cooperating kernels writes them
+        if (take_all || DIST_VALU) {      // exactly one of the two bodies writes them
 #pragma unroll
             for (int b = 0; b < GA_QB; ++b) {
                 if (!q_in[b]) continue;
@@ -657,6 +658,43 @@ void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     }
 }
 
+// One distance path for the whole grid ...
+template <bool DIST_VALU, bool LEGACY, int GA_QB>
+__global__ __launch_bounds__(GA_THREADS, 2)
+void geo_attn_fwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                         const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                         const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                         float* __restrict__ O, float* __restrict__ L,
+                         const int H, const int N, const int ZH, const int n_qtiles,
+                         const float* __restrict__ beta, const float min_rbf, const float max_rbf, const GaStrides st)
+{
+    __shared__ Smem sm;
+    geo_attn_fwd_body<DIST_VALU, LEGACY, GA_QB>(sm, (int)blockIdx.x, Q, K, V, coords, sigma, key_pad, O, L, H, N, ZH, n_qtiles, 1,
+                                                beta, min_rbf, max_rbf, st);
+}
+
+// ... or both over one grid of twice the size: workgroup g and workgroup n_wgs + g look at the same queries, the
+// first with the matrix-core distances, the second with the direct ones, and the one that does not own them
+// returns after the prologue.  One launch instead of two: the early exits overlap with the work.
+template <bool LEGACY, int GA_QB>
+__global__ __launch_bounds__(GA_THREADS, 2)
+void geo_attn_fwd_both_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                              const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                              const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                              float* __restrict__ O, float* __restrict__ L,
+                              const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs,
+                              const float* __restrict__ beta, const float min_rbf, const float max_rbf, const GaStrides st)
+{
+    __shared__ Smem sm;
+    const int id = (int)blockIdx.x;
+    if (id < n_wgs)
+        geo_attn_fwd_body<false, LEGACY, GA_QB>(sm, id, Q, K, V, coords, sigma, key_pad, O, L, H, N, ZH, n_qtiles, 0,
+                                                beta, min_rbf, max_rbf, st);
+    else
+        geo_attn_fwd_body<true, LEGACY, GA_QB>(sm, id - n_wgs, Q, K, V, coords, sigma, key_pad, O, L, H, N, ZH, n_qtiles, 0,
+                                               beta, min_rbf, max_rbf, st);
+}
+
 struct GaVariant { const char* name; };
 const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
@@ -694,15 +732,18 @@ int launch_attn_qb(const uint16_t* Q, const uint16_t* K, const uint16_t* V, cons
     constexpr int BM = GA_WAVES * 32 * QB;
     const int n_qtiles = (N + BM - 1) / BM;
     const int ZH = Z * H;
-    dim3 grid((unsigned)n_qtiles * (unsigned)ZH, 1, 1);
-    // dist 0: each workgroup picks its distance path (two launches over the same grid, see the kernel);
+    const unsigned n_wgs = (unsigned)n_qtiles * (unsigned)ZH;
+    // dist 0: each workgroup picks its distance path (one launch over twice the grid, see the kernel);
     // 1 / 2: force the matrix-core / vector-ALU path everywhere
-    if (dist != 2)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 1 ? 1 : 0, beta, min_rbf, max_rbf, gs);
-    if (dist != 1)
-        hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY, QB>), grid, dim3(GA_THREADS), 0, st,
-                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, dist == 2 ? 1 : 0, beta, min_rbf, max_rbf, gs);
+    if (dist == 0)
+        hipLaunchKernelGGL((geo_attn_fwd_both_kernel<LEGACY, QB>), dim3(2 * n_wgs), dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, beta, min_rbf, max_rbf, gs);
+    else if (dist == 1)
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<false, LEGACY, QB>), dim3(n_wgs), dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, beta, min_rbf, max_rbf, gs);
+    else
+        hipLaunchKernelGGL((geo_attn_fwd_kernel<true, LEGACY, QB>), dim3(n_wgs), dim3(GA_THREADS), 0, st,
+                           Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, beta, min_rbf, max_rbf, gs);
     return (int)hipGetLastError();
 }
 
