@@ -302,7 +302,7 @@ def main():
         torch.cuda.synchronize()
         b_ms = sum(e0.elapsed_time(e1) for e0, e1 in bev) / len(bev)
         result["geo_attn_bwd"] = {
-            "workload": "geometric attention backward, same shape: dQ, dK, dV, d_sigma (two launches, S and dP recomputed in each)",
+            "workload": "geometric attention backward, same shape: dQ, dK, dV, d_sigma (two passes in one launch, S and dP recomputed in each)",
             "ms": b_ms, "tflops_5_products": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12,
             "tflops_issued_7_products": 14.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12, "dtype": "bf16",
         }

@@ -11,7 +11,8 @@
 //   LEGACY logits  t = S + beta Rn |S|, Rn = 2 (rbf - min)/(max - min) - 1   (:448-449):
 //                  dt/dS = 1 + beta Rn sign(S), dt/drbf = 2 beta |S|/(max - min), d beta_h = sum dt Rn |S|  (:468-479)
 //
-// Two launches instead of the reference's one kernel with atomic adds into dQ (:501-503):
+// Two passes instead of the reference's one kernel with atomic adds into dQ (:501-503), run by the two
+// halves of one launch:
 //   OWN_Q = false  a wave owns 32 keys, streams the queries, accumulates dK, dV (and d sigma, d beta);
 //   OWN_Q = true   a wave owns 32 queries, streams the keys, accumulates dQ.
 // Both are the same code.  Scores are computed with the rows of the streamed ("other") tokens in the
@@ -64,17 +65,17 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
 struct GbStrides { long q[3], k[3], v[3], g[3], dq[3], dk[3], dv[3]; };
 
 template <bool OWN_Q, bool LEGACY>
-__global__ __launch_bounds__(GB_THREADS, 2)
-void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
-                         const uint16_t* __restrict__ V, const uint16_t* __restrict__ dO,
-                         const float* __restrict__ coords, const float* __restrict__ sigma,
-                         const float* __restrict__ beta, const uint8_t* __restrict__ key_pad,
-                         const float* __restrict__ Lse, const float* __restrict__ Dvec,
-                         float* __restrict__ dQ, float* __restrict__ dK, float* __restrict__ dV,
-                         float* __restrict__ d_sigma, float* __restrict__ d_beta,
-                         const int H, const int N, const int n_otiles, const float min_rbf, const float max_rbf, const GbStrides st)
+__device__ __forceinline__
+void geo_attn_bwd_body(BwdSmem& sm, const int block_id,
+                       const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                       const uint16_t* __restrict__ V, const uint16_t* __restrict__ dO,
+                       const float* __restrict__ coords, const float* __restrict__ sigma,
+                       const float* __restrict__ beta, const uint8_t* __restrict__ key_pad,
+                       const float* __restrict__ Lse, const float* __restrict__ Dvec,
+                       float* __restrict__ dQ, float* __restrict__ dK, float* __restrict__ dV,
+                       float* __restrict__ d_sigma, float* __restrict__ d_beta,
+                       const int H, const int N, const int n_otiles, const float min_rbf, const float max_rbf, const GbStrides& st)
 {
-    __shared__ BwdSmem sm;
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -82,8 +83,8 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     const int half = lane >> 5;
     const int col  = lane & 31;
 
-    const int ot = blockIdx.x % n_otiles;
-    const int zh = blockIdx.x / n_otiles;
+    const int ot = block_id % n_otiles;
+    const int zh = block_id / n_otiles;
     const int z  = zh / H;
     const int h  = zh - z * H;
     const size_t lin_off = (size_t)zh * (size_t)N;         // L and D are contiguous [Z,H,N]
@@ -408,6 +409,30 @@ void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restr
     }
 }
 
+// Both passes in one launch over twice the grid: workgroups [0, n_wgs) own keys (dK, dV, d sigma, d beta),
+// workgroups [n_wgs, 2 n_wgs) own queries (dQ).  The passes are independent, so one fills the other's tail.
+template <bool LEGACY>
+__global__ __launch_bounds__(GB_THREADS, 2)
+void geo_attn_bwd_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                         const uint16_t* __restrict__ V, const uint16_t* __restrict__ dO,
+                         const float* __restrict__ coords, const float* __restrict__ sigma,
+                         const float* __restrict__ beta, const uint8_t* __restrict__ key_pad,
+                         const float* __restrict__ Lse, const float* __restrict__ Dvec,
+                         float* __restrict__ dQ, float* __restrict__ dK, float* __restrict__ dV,
+                         float* __restrict__ d_sigma, float* __restrict__ d_beta,
+                         const int H, const int N, const int n_otiles, const int n_wgs,
+                         const float min_rbf, const float max_rbf, const GbStrides st)
+{
+    __shared__ BwdSmem sm;
+    const int id = (int)blockIdx.x;
+    if (id < n_wgs)
+        geo_attn_bwd_body<false, LEGACY>(sm, id, Q, K, V, dO, coords, sigma, beta, key_pad, Lse, Dvec, dQ, dK, dV, d_sigma, d_beta,
+                                         H, N, n_otiles, min_rbf, max_rbf, st);
+    else
+        geo_attn_bwd_body<true, LEGACY>(sm, id - n_wgs, Q, K, V, dO, coords, sigma, beta, key_pad, Lse, Dvec, dQ, dK, dV, d_sigma, d_beta,
+                                        H, N, n_otiles, min_rbf, max_rbf, st);
+}
+
 template <bool LEGACY>
 int launch_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
                const float* coords, const float* sigma, const float* beta, const uint8_t* mask,
@@ -415,11 +440,10 @@ int launch_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const ui
                int Z, int H, int N, float min_rbf, float max_rbf, const GbStrides& gs, hipStream_t st)
 {
     const int n_otiles = (N + GB_OWN - 1) / GB_OWN;
-    dim3 grid((unsigned)n_otiles * (unsigned)(Z * H), 1, 1);
-    hipLaunchKernelGGL((geo_attn_bwd_kernel<false, LEGACY>), grid, dim3(GB_THREADS), 0, st,
-                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf, gs);
-    hipLaunchKernelGGL((geo_attn_bwd_kernel<true, LEGACY>), grid, dim3(GB_THREADS), 0, st,
-                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, min_rbf, max_rbf, gs);
+    const unsigned n_wgs = (unsigned)n_otiles * (unsigned)(Z * H);
+    hipLaunchKernelGGL((geo_attn_bwd_kernel<LEGACY>), dim3(2 * n_wgs), dim3(GB_THREADS), 0, st,
+                       Q, K, V, dO, coords, sigma, beta, mask, L, D, dQ, dK, dV, d_sigma, d_beta, H, N, n_otiles, (int)n_wgs,
+                       min_rbf, max_rbf, gs);
     return (int)hipGetLastError();
 }
 
