@@ -27,8 +27,8 @@ H100_REFERENCE_GPW = 6.87194767e10 / 0.386 / 1e9   # README.md:34: 386 ms at thi
 # HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), bytes
 # WE: FETCH_SIZE 4370.5 KiB x 2.0 (calibration factor of that counter) + WRITE_SIZE 82271.9 KiB x 1.0
 WE_TRAFFIC_BYTES = int((4370.5 * 2.0 + 82271.9) * 1024)
-# attention: FETCH_SIZE (42510.3 + 830.6) KiB x 2.0 (both distance-path bodies of a call) + WRITE_SIZE 33280.0 KiB x 1.0
-ATTN_TRAFFIC_BYTES = int(((42510.3 + 830.6) * 2.0 + 33280.0) * 1024)
+# attention: FETCH_SIZE 43028.5 KiB x 2.0 (both distance-path bodies of the one launch) + WRITE_SIZE 33792.0 KiB x 1.0
+ATTN_TRAFFIC_BYTES = int((43028.5 * 2.0 + 33792.0) * 1024)
 
 
 def median(xs):
