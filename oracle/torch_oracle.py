@@ -166,20 +166,26 @@ def geo_attn_autograd_torch(Q, K, V, coords, sigma, key_padding_mask=None, betas
     """The dense statements above in a form torch.autograd can differentiate in Q, K, V, sigma and betas
     (the oracle of the backward kernel: nothing of the hand-derived gradient formulas enters here).
     betas=None: logits S*(1+rbf); otherwise the reference's S + b*rbf_norm*|S| with its pair mask.
-    Rows without any unmasked pair give O = 0 and pass no gradient."""
+    Rows without any unmasked pair give O = 0 and pass no gradient.
+    sigma (and betas) may also be given per query row, [Z,H,N]: the gradient with respect to such a tensor is the
+    contribution of every query row to the per-head gradient (their sum over Z and N), which tells how much of
+    the per-head number is left after cancellation."""
     Q, K, V = Q.to(dtype), K.to(dtype), V.to(dtype)
     coords, sigma = coords.to(dtype), sigma.to(dtype)
     Z, H, N, d = Q.shape
     mask = torch.zeros(Z, N, dtype=torch.bool) if key_padding_mask is None else key_padding_mask.bool()
     S = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(d)
     d2 = torch.sum((coords[:, :, None, :] - coords[:, None, :, :]) ** 2, dim=3)[:, None, :, :]
-    rbf = torch.exp(-d2 / (2 * sigma[None, :, None, None] ** 2))
+    sg = sigma[:, :, :, None] if sigma.dim() == 3 else sigma[None, :, None, None]
+    rbf = torch.exp(-d2 / (2 * sg ** 2))
     am = (mask[:, None, :, None] | mask[:, None, None, :]).expand(Z, H, N, N)
     if betas is None:
         T = S * (1 + rbf)
     else:
         am = am | (rbf < min_rbf) | (rbf > max_rbf)
-        T = S + betas.to(dtype)[None, :, None, None] * ((2 * (rbf - min_rbf) / (max_rbf - min_rbf)) - 1) * torch.abs(S)
+        bt = betas.to(dtype)
+        bt = bt[:, :, :, None] if bt.dim() == 3 else bt[None, :, None, None]
+        T = S + bt * ((2 * (rbf - min_rbf) / (max_rbf - min_rbf)) - 1) * torch.abs(S)
     T = torch.where(am, torch.full_like(T, float("-inf")), T)
     row_any = (~am).any(dim=-1, keepdim=True)
     T = torch.where(row_any, T, torch.zeros_like(T))

@@ -3,7 +3,15 @@ autograd function, against torch.autograd through the dense fp64 statement of th
 bf16-rounded inputs.
 
 Bar: the operands of every matrix product are bf16 (Q, K, V, dO, P, dS; the reference uses fp16), so each
-gradient tensor is compared in relative L2 norm: <= 1e-2 for dQ, dK, dV, d_sigma, d_beta (measured: 2.4e-3)."""
+gradient tensor is compared in relative L2 norm: <= 1e-2 for dQ, dK, dV (measured: 2.4e-3).
+
+The per-head scalars d_sigma and d_beta are sums over all pairs of terms of both signs, each carrying dP - D with
+D = rowsum(O * dO) from the forward's bf16 probabilities.  Where the per-query contributions cancel to a small
+remainder the relative error of that remainder measures the cancellation, not the kernel, so they are held to
+  |got - ref| <= 1e-2 * (sum over queries of |contribution of the query|)        always, and
+  relative L2 <= 1e-2                                                           where at least a quarter of that
+                                                                                 mass survives the cancellation.
+The oracle yields the per-query contributions as the gradient with respect to a per-query copy of sigma / beta."""
 import numpy as np
 import pytest
 import torch
@@ -37,12 +45,26 @@ def make(seed, Z, H, N, maskfrac=0.0, qscale=1.0):
 
 
 def reference_grads(Q, K, V, dO, coords, sigma, mask, betas=None, min_rbf=0.0, max_rbf=1.0):
+    """dQ, dK, dV and the per-query contributions [Z,H,N] to d_sigma and d_beta (their sums over Z and N are the
+    per-head gradients)."""
+    Z, H, N, _ = Q.shape
     q, k, v = (t.double().requires_grad_(True) for t in (Q, K, V))
-    s = sigma.double().requires_grad_(True)
-    b = None if betas is None else betas.double().requires_grad_(True)
+    s = sigma.double()[None, :, None].expand(Z, H, N).clone().requires_grad_(True)
+    b = None if betas is None else betas.double()[None, :, None].expand(Z, H, N).clone().requires_grad_(True)
     O = torch_oracle.geo_attn_autograd_torch(q, k, v, coords, s, mask, b, min_rbf, max_rbf)
     O.backward(dO.double())
     return q.grad, k.grad, v.grad, s.grad, None if b is None else b.grad
+
+
+def check_head_scalar(got, per_query, what):
+    total = per_query.sum(dim=(0, 2))
+    mass = per_query.abs().sum(dim=(0, 2))
+    err = (got.double() - total).abs()
+    assert torch.isfinite(got).all(), f"{what}: non-finite"
+    assert (err <= REL_L2_TOL * mass + 1e-9).all(), f"{what}: error / mass {(err / mass.clamp_min(1e-300)).max():.3e}"
+    if (total.abs() >= 0.25 * mass).all():
+        e = rel_l2(got.numpy(), total.numpy())
+        assert e <= REL_L2_TOL, f"{what}: rel-L2 {e:.3e}"
 
 
 def gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask, betas=None, min_rbf=0.0, max_rbf=1.0):
@@ -58,6 +80,9 @@ def gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask, betas=None, min_rbf=0.0, ma
 def compare(got, ref, mask, what):
     for g, r, name in zip(got, ref, ("dQ", "dK", "dV", "d_sigma", "d_beta")):
         if r is None:
+            continue
+        if name in ("d_sigma", "d_beta"):
+            check_head_scalar(g, r, f"{what} {name}")
             continue
         assert torch.isfinite(g).all(), f"{what} {name}: non-finite"
         e = rel_l2(g.numpy(), r.numpy())
