@@ -176,3 +176,27 @@ def test_differentiable_statement_equals_the_tiled_ones():
     torch_oracle.geo_attn_autograd_torch(q, K, V, coords, s, mask).sum().backward()
     assert torch.isfinite(q.grad).all() and torch.isfinite(s.grad).all()
     assert (q.grad[mask[:, None, :].expand(-1, H, -1)] == 0).all()
+
+
+def test_per_query_sigma_and_beta_split_the_per_head_gradients():
+    """sigma / beta given per query row [Z,H,N]: the same output, and gradients that sum over the queries to the
+    per-head ones (they are the per-query contributions the GPU tests weigh the per-head numbers against)."""
+    g = torch.Generator().manual_seed(12)
+    Z, H, N = 2, 3, 37
+    Q, K, V, dO = (torch.randn(Z, H, N, 64, generator=g, dtype=torch.float64) for _ in range(4))
+    coords = torch.cumsum(torch.randn(Z, N, 3, generator=g, dtype=torch.float64) * 2.2, dim=1)
+    mask = torch.rand(Z, N, generator=g) < 0.2
+    for betas, lo, hi in ((None, 0.0, 1.0), (torch.tensor([0.3, 1.0, 1.7], dtype=torch.float64), 0.05, 0.9)):
+        s_head = torch.tensor([2.0, 5.0, 11.0], dtype=torch.float64, requires_grad=True)
+        b_head = None if betas is None else betas.clone().requires_grad_(True)
+        O1 = torch_oracle.geo_attn_autograd_torch(Q, K, V, coords, s_head, mask, b_head, lo, hi)
+        O1.backward(dO)
+        s_rows = s_head.detach()[None, :, None].expand(Z, H, N).clone().requires_grad_(True)
+        b_rows = None if betas is None else betas[None, :, None].expand(Z, H, N).clone().requires_grad_(True)
+        O2 = torch_oracle.geo_attn_autograd_torch(Q, K, V, coords, s_rows, mask, b_rows, lo, hi)
+        O2.backward(dO)
+        assert torch.equal(O1.detach(), O2.detach())
+        assert torch.allclose(s_rows.grad.sum(dim=(0, 2)), s_head.grad, rtol=1e-10, atol=1e-12)
+        assert (s_rows.grad[mask[:, None, :].expand(Z, H, N)] == 0).all()          # a padded query contributes nothing
+        if betas is not None:
+            assert torch.allclose(b_rows.grad.sum(dim=(0, 2)), b_head.grad, rtol=1e-10, atol=1e-12)
