@@ -6,7 +6,8 @@
 //   O_i  = softmax_j(s_ij) V_j,  L_i = logsumexp_j s_ij;  padded/empty rows -> O = 0, L = -inf
 //
 // Mapping to the machine.  A workgroup is 4 waves; a wave owns 64 queries of one
-// (batch, head) as two blocks of 32 and walks the keys in tiles of 64 that the
+// (batch, head) as two blocks of 32 (one block where the grid would otherwise leave
+// half of the wave slots empty) and walks the keys in tiles of 64 that the
 // workgroup stages in LDS (K row-major, V transposed, key geometry), two tiles
 // deep: tile t is consumed while tile t+1 travels global -> registers -> LDS.
 // All products run on the matrix cores and are computed TRANSPOSED:
@@ -14,14 +15,15 @@
 //   D^T (keys x queries)  = G_tile (A, from LDS) x G_q^T (B, registers)     [geometry, see below]
 //   O^T (d x queries)    += V^T_tile (A, from LDS) x P^T (B, registers)
 // In the 32x32 accumulator layout a lane holds 16 rows of ONE column, so with
-// queries on the columns each lane owns one query per block: the row maximum,
-// the exponentials and the row sum are in-lane except for one exchange between
-// the two half-waves, and the S^T accumulator registers are, after conversion
+// queries on the columns each lane owns one query per block: the exponentials
+// and the row sum are in-lane (the two half-waves of a query meet only when its
+// softmax reference is re-based and at the end), and the S^T accumulator registers are, after conversion
 // to bf16, already the B operand of the last product (the contraction index is
 // merely visited in the permuted order the accumulator layout dictates, and the
 // V^T operand is read from LDS in that same order).  Every A fragment read from
-// LDS serves both query blocks, and the two blocks give the wave independent
-// matrix and vector work to overlap.
+// LDS serves both query blocks.  The softmax keeps a lazy reference instead of a
+// running maximum, and for blocks whose multiplier is 1 that reference is carried
+// into the score product as one more contraction slot (see the key loop).
 //
 // Geometry on the matrix cores.  With x' = (x - c) * sqrt(log2(e)/2)/sigma_h (c = a
 // point near the workgroup's queries) the multiplier is 1 + exp2(D),
