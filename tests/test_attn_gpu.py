@@ -169,6 +169,28 @@ def test_strided_operands_and_token_major_output_are_read_and_written_in_place(g
     assert torch.equal(O3, ref_O)
 
 
+def test_strided_output_rows_leave_the_gaps_between_them_alone(gpu):
+    """Raw C ABI: O with a token stride of 80 floats and L next to canaries: only the 64 floats of each row are
+    written, whatever the rows are embedded in."""
+    import ctypes
+    lib = _lib.load()
+    Z, H, N = 1, 2, 150
+    Q, K, V, coords, sigma, mask = make(33, Z, H, N, maskfrac=0.1)
+    q, k, v, c, s, m = (t.to(gpu) for t in (Q, K, V, coords, sigma, mask.view(torch.uint8)))
+    ref = pa.geo_attn(q, k, v, c, s, mask.to(gpu))
+    buf = torch.full((Z, H, N, 80), -7.25, device=gpu)
+    Lb = torch.full((Z * H * N + 32,), -7.25, device=gpu)
+    plain = [H * N * 64, N * 64, 64]
+    strides = (ctypes.c_int64 * 12)(*(plain * 3 + [H * N * 80, N * 80, 80]))
+    rc = lib.proteus_geo_attn_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), strides, c.data_ptr(), s.data_ptr(),
+                                          m.data_ptr(), buf.data_ptr(), Lb.data_ptr(), Z, H, N, 64, 0,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(buf[..., :64], ref)
+    assert (buf[..., 64:] == -7.25).all() and (Lb[Z * H * N:] == -7.25).all()
+
+
 def test_flat_multiplier_equals_sdpa_on_gpu(gpu):
     # sigma -> infinity: multiplier == 2 -> torch SDPA with scale 2/sqrt(d), evaluated in fp32 on the same bf16 values
     Q, K, V, coords, _, _ = make(3, 2, 4, 777)
