@@ -292,6 +292,13 @@ int proteus_geo_attn_fwd_strided_check(const uint16_t* Q, const uint16_t* K, con
                                        const float* coords, const float* sigma, const uint8_t* key_pad_mask,
                                        const float* O, const float* L,
                                        int Z, int H, int N, int d_head, int tuning);
+int proteus_geo_attn_legacy_fwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                        const int64_t* strides,
+                                        const float* coords, const float* sigma, const float* beta,
+                                        const uint8_t* key_pad_mask,
+                                        float* O, float* L,
+                                        int Z, int H, int N, int d_head,
+                                        float min_rbf, float max_rbf, int tuning, void* stream);
 int proteus_geo_attn_bwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
                                  const int64_t* strides,
                                  const float* coords, const float* sigma, const float* beta,

@@ -20,6 +20,7 @@ SYMBOLS = [
     "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
     "proteus_geo_attn_bwd_check", "proteus_geo_attn_fwd_strided", "proteus_geo_attn_fwd_strided_check",
+    "proteus_geo_attn_legacy_fwd_strided",
     "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_probe_valu_rate", "proteus_probe_sincos",
@@ -88,6 +89,9 @@ def load():
     lib.proteus_geo_attn_fwd_strided.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     lib.proteus_geo_attn_fwd_strided_check.restype = ci
     lib.proteus_geo_attn_fwd_strided_check.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
+    lib.proteus_geo_attn_legacy_fwd_strided.restype = ci
+    lib.proteus_geo_attn_legacy_fwd_strided.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci,
+                                                        ctypes.c_float, ctypes.c_float, ci, vp]
     lib.proteus_geo_attn_bwd_strided.restype = ci
     lib.proteus_geo_attn_bwd_strided.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, vp]
     lib.proteus_geo_attn_bwd_strided_check.restype = ci

@@ -846,3 +846,23 @@ extern "C" int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K,
     return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf, contiguous_strides(H, N),
                              reinterpret_cast<hipStream_t>(stream));
 }
+
+extern "C" int proteus_geo_attn_legacy_fwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                                   const int64_t* strides,
+                                                   const float* coords, const float* sigma, const float* beta,
+                                                   const uint8_t* key_pad_mask,
+                                                   float* O, float* L,
+                                                   int Z, int H, int N, int d_head,
+                                                   float min_rbf, float max_rbf, int tuning, void* stream)
+{
+    int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    if (!beta) return PROTEUS_ERR_NULL_POINTER;
+    if (!(max_rbf > min_rbf)) return PROTEUS_ERR_BAD_SHAPE;
+    GaStrides gs;
+    rc = strides_from(strides, Z, H, N, gs);
+    if (rc != PROTEUS_OK) return rc;
+    if ((tuning == 0 || tuning >= 3) && (min_rbf > 0.f || max_rbf < 1.f)) tuning = 2;
+    return launch_attn<true>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, beta, min_rbf, max_rbf, gs,
+                             reinterpret_cast<hipStream_t>(stream));
+}

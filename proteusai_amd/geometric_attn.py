@@ -74,10 +74,7 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     lib = _lib.load()
     dev = Q.device
     legacy = betas is not None
-    if legacy:      # the beta-weighted logits have no strided entry point
-        q, k, v = (t.detach().to(torch.bfloat16).contiguous() for t in (Q, K, V))
-    else:
-        q, k, v = _operand(Q), _operand(K), _operand(V)
+    q, k, v = _operand(Q), _operand(K), _operand(V)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
     m = None
@@ -85,7 +82,7 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         if tuple(key_padding_mask.shape) != (Z, N):
             raise AssertionError(f"mask must be of shape ({Z}, {N}), not {tuple(key_padding_mask.shape)}")
         m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
-    if token_major_out and not legacy:
+    if token_major_out:
         O = torch.empty(Z, N, H, d, dtype=torch.float32, device=dev).permute(0, 2, 1, 3)
     else:
         O = torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
@@ -106,10 +103,17 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
             if betas.dim() != 1 or betas.size(0) != H:
                 raise AssertionError(f"number of betas must be equal to nheads, not {tuple(betas.shape)} and {H=}")
             bt = betas.detach().to(device=dev, dtype=torch.float32).contiguous()
-            rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
-                                                 bt.data_ptr(), None if m is None else m.data_ptr(),
-                                                 O.data_ptr(), L.data_ptr(), Z, H, N, d,
-                                                 float(min_rbf), float(max_rbf), int(tuning), stream)
+            if _is_plain(q, k, v, O):
+                rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
+                                                     bt.data_ptr(), None if m is None else m.data_ptr(),
+                                                     O.data_ptr(), L.data_ptr(), Z, H, N, d,
+                                                     float(min_rbf), float(max_rbf), int(tuning), stream)
+            else:
+                rc = lib.proteus_geo_attn_legacy_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                             _lib.stride_array(q, k, v, O), c.data_ptr(), s.data_ptr(),
+                                                             bt.data_ptr(), None if m is None else m.data_ptr(),
+                                                             O.data_ptr(), L.data_ptr(), Z, H, N, d,
+                                                             float(min_rbf), float(max_rbf), int(tuning), stream)
     _lib.check(rc, "proteus_geo_attn_fwd")
     return (O, L) if return_lse else O
 
@@ -265,7 +269,7 @@ class GeoAttention(nn.Module):
         # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
         if self.legacy_logits:
             out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf,
-                                 max_rbf=self.max_rbf, check_spreads=False, out_dtype=q.dtype)
+                                 max_rbf=self.max_rbf, check_spreads=False, token_major_out=True, out_dtype=q.dtype)
         else:
             out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False,
                                  token_major_out=True, out_dtype=q.dtype)

@@ -70,7 +70,7 @@ def test_attention_forward_and_backward(gpu, case):
 
     s = sigma.to(gpu).requires_grad_(True)
     bt = None if betas is None else betas.to(gpu).requires_grad_(True)
-    strided = (not legacy) and case % 2 == 1
+    strided = case % 2 == 1
     what += f" strided={strided}"
     if strided:
         # operands as slices of one fused [Z,N,3,H,d] buffer, O token-major: read and written in place
