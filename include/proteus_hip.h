@@ -35,6 +35,7 @@ extern "C" {
 #define PROTEUS_ERR_BAD_ALIGNMENT -5   /* a pointer is not aligned as required    */
 #define PROTEUS_ERR_BAD_TUNING    -6   /* unknown tuning/variant selector         */
 #define PROTEUS_ERR_UNSUPPORTED   -7   /* legacy option not implemented           */
+#define PROTEUS_ERR_TOO_LARGE     -8   /* beyond the fixed capacity of an entry point that allocates nothing */
 
 /* ---- coordinate layouts accepted by proteus_we_fwd ---- */
 #define PROTEUS_COORDS_SOA 0   /* [Z,3,N]: what the reference's wrapper hands its kernel */
@@ -44,6 +45,7 @@ extern "C" {
 #define PROTEUS_WE_MAX_N   (1 << 22)
 #define PROTEUS_WE_MAX_K   4096
 #define PROTEUS_ATTN_MAX_N (1 << 20)
+#define PROTEUS_WE_BWD_STATIC_MAX_K 512   /* most wavenumbers proteus_we_bwd_static takes */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int proteus_version(void);
@@ -176,6 +178,21 @@ int proteus_we_bwd(const float* d_out, const float* cos_sums, const float* sin_s
 int proteus_we_bwd_check(const float* d_out, const float* cos_sums, const float* sin_sums,
                          const float* d_wavenumbers, const float* workspace, size_t workspace_bytes,
                          int Z, int N, int K);
+
+/*
+ * proteus_we_bwd for callers that cannot allocate device memory or hand over a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Same kernels and the same,
+ * bit-identical result as proteus_we_bwd; the partial sums live in a 2 MiB array in
+ * the library's own device image instead of a workspace, which every GPU the library
+ * runs on holds until the process ends.  Calls no hipMalloc / hipFree.
+ *   K > PROTEUS_WE_BWD_STATIC_MAX_K returns PROTEUS_ERR_TOO_LARGE (before any HIP call).
+ *   The GPU that is current at the call must be the one `stream` belongs to.
+ *   All calls on one GPU share that GPU's array: calls that overlap there (two
+ *   streams, two threads) race; serialise them.  Nothing has to be cleared between calls.
+ */
+int proteus_we_bwd_static(const float* d_out, const float* cos_sums, const float* sin_sums,
+                          float* d_wavenumbers, int Z, int N, int K, void* stream);
 
 int proteus_we_aniso_bwd(const float* d_out, const float* d_cb, const float* d_k,
                          float* g_cb, float* g_k, float* workspace, size_t workspace_bytes,

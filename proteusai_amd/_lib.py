@@ -17,7 +17,7 @@ SYMBOLS = [
     "proteus_version", "proteus_strerror",
     "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_num_variants", "proteus_we_variant_name",
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
-    "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
+    "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_bwd_static", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
     "proteus_geo_attn_bwd_check", "proteus_geo_attn_fwd_strided", "proteus_geo_attn_fwd_strided_check",
     "proteus_geo_attn_legacy_fwd_strided",
@@ -68,6 +68,8 @@ def load():
     lib.proteus_we_bwd_workspace_bytes.argtypes = [ci, ci, ci]
     lib.proteus_we_bwd.restype = ci
     lib.proteus_we_bwd.argtypes = [vp, vp, vp, vp, vp, sz, ci, ci, ci, vp]
+    lib.proteus_we_bwd_static.restype = ci
+    lib.proteus_we_bwd_static.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     lib.proteus_we_bwd_check.restype = ci
     lib.proteus_we_bwd_check.argtypes = [vp, vp, vp, vp, vp, sz, ci, ci, ci]
     lib.proteus_we_aniso_bwd.restype = ci

@@ -360,6 +360,7 @@ extern "C" const char* proteus_strerror(int code) {
         case PROTEUS_ERR_BAD_ALIGNMENT: return "a pointer is not 16-byte aligned";
         case PROTEUS_ERR_BAD_TUNING:    return "unknown tuning selector";
         case PROTEUS_ERR_UNSUPPORTED:   return "option not implemented";
+        case PROTEUS_ERR_TOO_LARGE:     return "size beyond the fixed capacity of this entry point";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

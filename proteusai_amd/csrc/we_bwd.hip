@@ -12,7 +12,13 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 #include "proteus_hip.h"
+
+// Partial sums of proteus_we_bwd_static: one row of PROTEUS_WE_BWD_STATIC_MAX_K floats per slab (2 MiB).  Every
+// GPU the library runs on holds its own copy at its own address until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+static __device__ __align__(256) float scratch[1024 * PROTEUS_WE_BWD_STATIC_MAX_K];
 
 namespace {
 
@@ -20,6 +26,7 @@ constexpr int WB_THREADS   = 256;
 constexpr int WB_MAX_SLABS = 1024;     // rows of partial sums in the workspace
 constexpr int WB_MIN_ROWS  = 8;        // a slab is not made smaller than this
 constexpr int WB_UNROLL    = 4;        // token rows in flight per lane
+static_assert(sizeof(scratch) == (size_t)WB_MAX_SLABS * PROTEUS_WE_BWD_STATIC_MAX_K * sizeof(float), "scratch holds one row per slab");
 
 __host__ __device__ inline int slabs_for(long rows) {
     long g = (rows + WB_MIN_ROWS - 1) / WB_MIN_ROWS;
@@ -174,6 +181,54 @@ extern "C" int proteus_we_bwd(const float* d_out, const float* cos_sums, const f
                        d_out, cos_sums, sin_sums, workspace, rows, K, 1);
     hipLaunchKernelGGL(we_bwd_final_kernel, dim3((K + WB_FK - 1) / WB_FK), dim3(WB_THREADS), 0, st,
                        (const float*)workspace, d_wavenumbers, (float*)nullptr, slabs, K, 1);
+    return (int)hipGetLastError();
+}
+
+namespace {
+
+// Device address of `scratch` on each GPU, looked up on the first call made with that GPU current.
+constexpr int WB_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+float*     g_scratch_ptr[WB_MAX_DEVICES] = {};
+
+int scratch_for_current_device(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= WB_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return PROTEUS_OK;
+}
+
+}  // namespace
+
+extern "C" int proteus_we_bwd_static(const float* d_out, const float* cos_sums, const float* sin_sums,
+                                     float* d_wavenumbers, int Z, int N, int K, void* stream)
+{
+    if (!d_out || !cos_sums || !sin_sums || !d_wavenumbers) return PROTEUS_ERR_NULL_POINTER;
+    if (Z <= 0 || N <= 0 || K <= 0 || N > PROTEUS_WE_MAX_N) return PROTEUS_ERR_BAD_SHAPE;
+    if (K > PROTEUS_WE_BWD_STATIC_MAX_K) return PROTEUS_ERR_TOO_LARGE;
+    if ((uintptr_t)d_out & 7) return PROTEUS_ERR_BAD_ALIGNMENT;
+    float* partial = nullptr;
+    const int rc = scratch_for_current_device(&partial);
+    if (rc != PROTEUS_OK) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const long rows = (long)Z * N;
+    const int slabs = slabs_for(rows);
+    const int kchunks = (K + WB_THREADS - 1) / WB_THREADS;
+    // the first kernel overwrites every partial sum the second one reads: nothing has to start at zero
+    hipLaunchKernelGGL((we_bwd_partial_kernel<false>), dim3(slabs, kchunks), dim3(WB_THREADS), 0, st,
+                       d_out, cos_sums, sin_sums, partial, rows, K, 1);
+    hipLaunchKernelGGL(we_bwd_final_kernel, dim3((K + WB_FK - 1) / WB_FK), dim3(WB_THREADS), 0, st,
+                       (const float*)partial, d_wavenumbers, (float*)nullptr, slabs, K, 1);
     return (int)hipGetLastError();
 }
 
