@@ -43,6 +43,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "proteus_hip.h"
 
 namespace {
@@ -660,6 +661,8 @@ void geo_attn_fwd_body(Smem& sm, const int block_id,
     }
 }
 
+#include "geo_attn_fwd_pipe.inc"
+
 // One distance path for the whole grid ...
 template <bool DIST_VALU, bool LEGACY, int GA_QB>
 __global__ __launch_bounds__(GA_THREADS, 2)
@@ -697,8 +700,31 @@ void geo_attn_fwd_both_kernel(const uint16_t* __restrict__ Q, const uint16_t* __
                                                beta, min_rbf, max_rbf, st);
 }
 
+// The pipelined body over the first half of a doubled grid, the direct-distance body (for workgroups whose
+// queries are spread too widely for the matrix-core distances) over the second; take_all: the pipelined body alone.
+__global__ __launch_bounds__(GA_THREADS, 2)
+void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                              const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                              const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                              float* __restrict__ O, float* __restrict__ L,
+                              const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs, const int take_all,
+                              const GaStrides st)
+{
+    extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
+    const int id = (int)blockIdx.x;
+    if (id < n_wgs)
+        geo_attn_fwd_pipe_body(*reinterpret_cast<PipeSmem*>(ga_dyn_smem), id, Q, K, V, coords, sigma, key_pad, O, L,
+                               H, N, ZH, n_qtiles, take_all, st);
+    else
+        geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), id - n_wgs, Q, K, V, coords, sigma, key_pad, O, L,
+                                          H, N, ZH, n_qtiles, 0, nullptr, 0.f, 1.f, st);
+}
+constexpr size_t GA_PIPE_LDS = sizeof(PipeSmem) > sizeof(Smem) ? sizeof(PipeSmem) : sizeof(Smem);
+static_assert(GA_PIPE_LDS <= 80 * 1024, "two workgroups per compute unit");
+
 struct GaVariant { const char* name; };
-const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"} };
+const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"},
+                                {"pipelined"}, {"pipelined_dist_mfma"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -749,18 +775,42 @@ int launch_attn_qb(const uint16_t* Q, const uint16_t* K, const uint16_t* V, cons
     return (int)hipGetLastError();
 }
 
+int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                     const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, bool take_all,
+                     const GaStrides& gs, hipStream_t st)
+{
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)GA_PIPE_LDS);
+    if (attr != hipSuccess) return (int)attr;
+    constexpr int BM = GA_WAVES * 64;
+    const int n_qtiles = (N + BM - 1) / BM;
+    const int ZH = Z * H;
+    const unsigned n_wgs = (unsigned)n_qtiles * (unsigned)ZH;
+    hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gs);
+    return (int)hipGetLastError();
+}
+
 template <bool LEGACY>
 int launch_attn(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                 const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
 {
     // Two query blocks per wave unless that leaves at most one workgroup per compute unit (256 of them on
-    // this chip, two workgroups each): then one block per wave doubles the waves in flight.
+    // this chip, two workgroups each): then one block per wave doubles the waves in flight.  With two blocks per
+    // wave the README logits take the software-pipelined kernel.
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
     bool one_block = wgs2 <= 256;
     int dist = tuning;
+    bool pipelined = !LEGACY && tuning == 0 && !one_block;
+    bool take_all = false;
     if (tuning == 3) { one_block = true;  dist = 0; }
     if (tuning == 4) { one_block = false; dist = 0; }
+    if (tuning == 5 || tuning == 6) {                   // the pipelined kernel whatever the grid (6: without the direct-distance body beside it)
+        if (LEGACY) { one_block = false; dist = 0; }
+        else { pipelined = true; take_all = (tuning == 6); }
+    }
+    if (pipelined) return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, take_all, gs, st);
     return one_block ? launch_attn_qb<LEGACY, 1>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, gs, st)
                      : launch_attn_qb<LEGACY, 2>(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, dist, beta, min_rbf, max_rbf, gs, st);
 }

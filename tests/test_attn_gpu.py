@@ -39,9 +39,14 @@ def make(seed, Z, H, N, qscale=1.0, maskfrac=0.0, tail=False):
     return Q, K, V, coords, sigma, mask
 
 
-def run_gpu(gpu, Q, K, V, coords, sigma, mask):
+# 0: the launcher's choice (small grids take the kernel with one query block per wave); 5: the software-pipelined
+# kernel, which large grids take, forced on these small shapes too (its direct-distance fallback beside it)
+KERNELS = [0, 5]
+
+
+def run_gpu(gpu, Q, K, V, coords, sigma, mask, tuning=0):
     O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu),
-                       None if mask is None else mask.to(gpu), return_lse=True)
+                       None if mask is None else mask.to(gpu), return_lse=True, tuning=tuning)
     torch.cuda.synchronize()
     return O.cpu().numpy(), L.cpu().numpy()
 
@@ -63,10 +68,11 @@ def check(got, Q, K, V, coords, sigma, mask, rows=None, what=""):
     return err
 
 
-@pytest.mark.parametrize("N", [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 513])
-def test_ragged_lengths(gpu, N):
+@pytest.mark.parametrize("tuning", KERNELS)
+@pytest.mark.parametrize("N", [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 200, 255, 256, 257, 513])
+def test_ragged_lengths(gpu, N, tuning):
     a = make(100 + N, 2, 3, N)
-    check(run_gpu(gpu, *a), *a, what=f"N={N}")
+    check(run_gpu(gpu, *a, tuning=tuning), *a, what=f"N={N}")
 
 
 def test_golden_fixture(gpu, golden_dir):
@@ -79,7 +85,8 @@ def test_golden_fixture(gpu, golden_dir):
     assert (O[~fin] == 0).all()
 
 
-def test_masks(gpu):
+@pytest.mark.parametrize("tuning", KERNELS)
+def test_masks(gpu, tuning):
     N = 300
     Q, K, V, coords, sigma, _ = make(1, 5, 2, N)
     g = torch.Generator().manual_seed(1)
@@ -90,18 +97,20 @@ def test_masks(gpu):
     mask[3] = True
     mask[3, 77] = False                              # one valid token
     mask[4, :64] = True                              # a whole leading key tile padded
-    check(run_gpu(gpu, Q, K, V, coords, sigma, mask), Q, K, V, coords, sigma, mask, what="masks")
+    check(run_gpu(gpu, Q, K, V, coords, sigma, mask, tuning=tuning), Q, K, V, coords, sigma, mask, what="masks")
 
 
-def test_large_logits(gpu):
+@pytest.mark.parametrize("tuning", KERNELS)
+def test_large_logits(gpu, tuning):
     # logits of order +-40: the online softmax must not overflow or lose the maximum
     a = make(2, 1, 4, 400, qscale=2.5)
-    check(run_gpu(gpu, *a), *a, what="large logits")
+    check(run_gpu(gpu, *a, tuning=tuning), *a, what="large logits")
 
 
 @pytest.mark.parametrize("profile", ["rising", "falling", "sawtooth", "late_spike", "very_negative_start", "masked_start"])
 @pytest.mark.parametrize("near", [False, True])
-def test_softmax_reference_is_rebased_when_the_scores_run_away(gpu, profile, near):
+@pytest.mark.parametrize("tuning", KERNELS)
+def test_softmax_reference_is_rebased_when_the_scores_run_away(gpu, profile, near, tuning):
     """Scores that climb, fall or jump by hundreds along the key axis: the kernel keeps a lazy softmax reference
     (no running maximum) and must re-base it exactly when an exponential would run away, whatever the order."""
     N, H = 640, 2
@@ -129,7 +138,7 @@ def test_softmax_reference_is_rebased_when_the_scores_run_away(gpu, profile, nea
         mask[0, :130] = True
         mask[0, 300:333] = True
     a = (Q, K, V, coords, sigma, mask)
-    check(run_gpu(gpu, *a), *a, what=f"{profile}, near={near}")
+    check(run_gpu(gpu, *a, tuning=tuning), *a, what=f"{profile}, near={near}")
 
 
 def test_every_variant_matches_the_oracle(gpu):
@@ -216,6 +225,28 @@ def test_key_padding_equals_truncation(gpu):
     O2, L2 = run_gpu(gpu, Q[:, :, :200].contiguous(), K[:, :, :200].contiguous(), V[:, :, :200].contiguous(),
                      coords[:, :200].contiguous(), sigma, None)
     assert np.array_equal(O[:, :, :200], O2) and np.array_equal(L[:, :, :200], L2)
+
+
+@pytest.mark.parametrize("tuning", KERNELS)
+def test_what_padded_tokens_hold_cannot_reach_valid_rows(gpu, tuning):
+    """NaN, Inf and huge values in Q, K, V and the coordinates of padded tokens: the valid rows come out bit for bit as
+    with zeros there, padded rows are exactly zero (scattered and tail padding; several key tiles)."""
+    Z, H, N = 2, 3, 450
+    Q, K, V, coords, sigma, mask = make(41, Z, H, N, maskfrac=0.15, tail=True)
+    clean = [t.clone() for t in (Q, K, V, coords)]
+    junk = torch.tensor([float("nan"), float("inf"), -float("inf"), 3e38, -1e30])
+    g = torch.Generator().manual_seed(41)
+    for t, c in zip((Q, K, V), clean[:3]):
+        pick = junk[torch.randint(0, 5, (Z, N), generator=g)].to(t.dtype)
+        t[:] = torch.where(mask[:, None, :, None], pick[:, None, :, None], t)
+        c[:] = torch.where(mask[:, None, :, None], torch.zeros((), dtype=t.dtype), c)
+    pick = junk[torch.randint(0, 5, (Z, N), generator=g)]
+    coords[:] = torch.where(mask[:, :, None], pick[:, :, None], coords)
+    clean[3][:] = torch.where(mask[:, :, None], torch.zeros(()), clean[3])
+    O1, L1 = run_gpu(gpu, Q, K, V, coords, sigma, mask, tuning=tuning)
+    O0, L0 = run_gpu(gpu, *clean, sigma, mask, tuning=tuning)
+    assert np.array_equal(O1, O0) and np.array_equal(L1, L0)
+    check((O0, L0), *clean, sigma, mask, what="padded junk")
 
 
 def test_rigid_motion_of_coordinates(gpu):
