@@ -49,7 +49,7 @@ def probe_rates(lib, torch, dev):
     """Measured lane-op rates (lane-ops/s) of the instructions the WE inner loop issues."""
     # scalar-operand forms (ops 0-2), transcendentals, and the vector-operand forms of the accumulations
     names = {0: "fma_s", 1: "mul_s", 2: "add_s", 3: "sin", 4: "cos", 5: "exp2", 6: "rsq", 7: "fract",
-             20: "fmac_v", 21: "add_v"}
+             8: "fmac_v", 9: "add_v"}
     sink = torch.empty(2048 * 256, device=dev)
     rates = {}
     for op, name in names.items():

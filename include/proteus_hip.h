@@ -7,8 +7,10 @@
  *
  * Conventions shared by every entry point
  *   - All pointers are DEVICE pointers owned by the caller; the library borrows
- *     them for the duration of the launch and keeps nothing.  Outputs are fully
- *     overwritten (no reliance on zero-initialisation, no atomics).
+ *     them for the duration of the launch and keeps nothing.  Tensor outputs are
+ *     fully overwritten (no reliance on zero-initialisation, no atomics).  The one
+ *     exception are the per-head scalars d_sigma and d_beta of proteus_geo_attn_bwd:
+ *     they are ACCUMULATED into with atomic adds and must be zeroed by the caller.
  *   - All tensors are dense and contiguous in the stated layout.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *     Launches are asynchronous; no entry point synchronises.
@@ -337,32 +339,12 @@ const char* proteus_geo_attn_variant_name(int tuning);
  * Instruction-rate probe used to state the roofline denominator of the WE
  * kernel.  Runs `iters` rounds of 64 independent chains of one VALU
  * instruction per lane on `blocks` x 256 threads and writes one float per
- * thread to `sink` (so the work cannot be removed).  The caller times the
- * launch; lane-ops issued = blocks*256*iters*64.  No counterpart in the
- * reference.
- *   op: 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_sin_f32, 4 v_cos_f32,
- *       5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32;
- *       8, 9, 10: one stream mixing 16 v_sin_f32 chains with 16, 32, 48 v_fma_f32
- *       chains (lane-ops issued = blocks*256*iters*(16 + 16|32|48)): whether the
- *       transcendental and the ordinary fp32 pipelines overlap;
- *       11, 12, 13: the same with a fixed program order, every v_sin_f32 followed
- *       by 1, 2, 3 v_fma_f32 (lane-ops = blocks*256*iters*16*(1 + 1|2|3));
- *       14: blocks/2 workgroups of 8 waves, four running 64 v_sin_f32 chains and four 64 v_fma_f32 chains
- *       (overlap across waves of one SIMD);
- *       15, 17: the embedding kernel's inner step on register data, 8 and 32
- *       wavenumbers per step (7 instructions each, two of them transcendental);
- *       16, 18: the same with the two transcendentals replaced by multiplies;
- *       19..22: 64 chains with vector-register operands only: x = fma(x,u,v),
- *       x = fma(u,v,x), x += u, x *= u (ops 0..2 feed scalar-register operands);
- *       23..26: blocks/2 workgroups of 8 waves, 16 links per lane and round of
- *       v_mfma_f32_4x4x1_16B_f32 alone, v_sin_f32 alone, both in one stream, and
- *       four waves of each kind (matrix pipeline beside the transcendental one);
- *       27..30: per link four v_mfma_f32_32x32x16_bf16 alone, 32 v_fmac_f32 alone,
- *       both in one stream, and the MFMAs with 32 v_exp_f32 in one stream;
- *       31..33: blocks/2 workgroups of 8 waves: waves 0-3 alone (four MFMAs per
- *       link), waves 4-7 alone (16 v_exp_f32 + 16 v_fmac_f32 per link), both kinds
- *       together (matrix and vector work in different waves of a SIMD);
- *       34: 64 chains of v_mul_f32 whose first source is a quad broadcast through DPP
+ * thread to `sink` (blocks * 256 floats; so the work cannot be removed).  The
+ * caller times the launch; lane-ops issued = blocks*256*iters*64.  No
+ * counterpart in the reference.
+ *   op: 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32 (second operand a scalar register),
+ *       3 v_sin_f32, 4 v_cos_f32, 5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32;
+ *       8 v_fmac_f32 and 9 v_add_f32 with vector-register operands only.
  */
 int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
 

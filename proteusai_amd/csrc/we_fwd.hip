@@ -207,23 +207,26 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
     // ---- epilogue: each lane writes its own rows ----
     const size_t row = zN + (size_t)i;
     float* o  = out      + row * (size_t)(2 * K) + 2 * (size_t)k0;
-    float* pc = cos_sums + row * (size_t)K + k0;
-    float* ps = sin_sums + row * (size_t)K + k0;
 
-    const float keep = i_valid ? 1.0f : 0.0f;    // padded observer: zeros
+    // padded observer: exact zeros, whatever its lane accumulated (its coordinates may hold anything, NaN included,
+    // so the sums are selected away, not multiplied by zero)
+    auto kept = [&](const float v) { return i_valid ? v : 0.0f; };
+    float* pc = nullptr;
+    float* ps = nullptr;
+    if (MAG != WE_MAG_NO_SUMS) { pc = cos_sums + row * (size_t)K + k0; ps = sin_sums + row * (size_t)K + k0; }
     if (k0 + KT <= K && (K & 1) == 0 && (KT & 3) == 0 && (K & 3) == 0) {
         // full tile, rows 16-byte aligned: vector stores
 #pragma unroll
         for (int t = 0; t < KT; t += 2) {
-            float4 v = make_float4(acc_oc[t] * keep, acc_os[t] * keep, acc_oc[t + 1] * keep, acc_os[t + 1] * keep);
+            float4 v = make_float4(kept(acc_oc[t]), kept(acc_os[t]), kept(acc_oc[t + 1]), kept(acc_os[t + 1]));
             *reinterpret_cast<float4*>(o + 2 * t) = v;
         }
 #pragma unroll
         for (int t = 0; t < KT; t += 4) {
             if (MAG == WE_MAG_NO_SUMS) break;
-            float4 c = make_float4((acc_c[t] - nzero) * keep, (acc_c[t + 1] - nzero) * keep,
-                                   (acc_c[t + 2] - nzero) * keep, (acc_c[t + 3] - nzero) * keep);
-            float4 s = make_float4(acc_s[t] * keep, acc_s[t + 1] * keep, acc_s[t + 2] * keep, acc_s[t + 3] * keep);
+            float4 c = make_float4(kept(acc_c[t] - nzero), kept(acc_c[t + 1] - nzero),
+                                   kept(acc_c[t + 2] - nzero), kept(acc_c[t + 3] - nzero));
+            float4 s = make_float4(kept(acc_s[t]), kept(acc_s[t + 1]), kept(acc_s[t + 2]), kept(acc_s[t + 3]));
             *reinterpret_cast<float4*>(pc + t) = c;
             *reinterpret_cast<float4*>(ps + t) = s;
         }
@@ -231,11 +234,11 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
             if (k0 + t < K) {
-                o[2 * t]     = acc_oc[t] * keep;
-                o[2 * t + 1] = acc_os[t] * keep;
+                o[2 * t]     = kept(acc_oc[t]);
+                o[2 * t + 1] = kept(acc_os[t]);
                 if (MAG == WE_MAG_NO_SUMS) continue;
-                pc[t] = (acc_c[t] - nzero) * keep;
-                ps[t] = acc_s[t] * keep;
+                pc[t] = kept(acc_c[t] - nzero);
+                ps[t] = kept(acc_s[t]);
             }
         }
     }

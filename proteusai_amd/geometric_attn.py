@@ -211,11 +211,15 @@ class GeoAttention(nn.Module):
     sigma = min_spread + exp(w), heads concatenated as a (d_k x heads)
     interleave, bias-free output projection).  With legacy_logits=True the
     logits are the reference module's (beta-weighted bias, [min_rbf, max_rbf]
-    pair mask); otherwise beta_weights is kept only so that state dicts line up."""
+    pair mask); otherwise beta_weights is kept only so that state dicts line up.
+    min_rbf=None takes the reference module's default 0.001 (encoder.py:57) with legacy_logits and 0 without
+    (the README logits have no pair mask)."""
 
-    def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=0.0, max_rbf=1.00, learn_spreads=True,
+    def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=None, max_rbf=1.00, learn_spreads=True,
                  legacy_logits=False):
         super().__init__()
+        if min_rbf is None:
+            min_rbf = 0.001 if legacy_logits else 0.0
         self.legacy_logits = legacy_logits      # True: the reference module's beta-weighted bias and pair mask
         self.heads = heads
         self.d_model = d_model

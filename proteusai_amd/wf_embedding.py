@@ -126,11 +126,15 @@ class _wf_embedding(torch.autograd.Function):
         out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type, need_sums=need)
         if need:
             ctx.save_for_backward(cos_sums, sin_sums)
+        ctx.need = need
         ctx.wn_dtype = wavenumbers.dtype
         return out
 
     @staticmethod
     def backward(ctx, dO):
+        # (autograd also comes here when only another input, e.g. the coordinates, asks for a gradient: there is none to give)
+        if not ctx.need:
+            return None, None, None, None, None
         cos_sums, sin_sums = ctx.saved_tensors
         dk = we_backward(dO, cos_sums, sin_sums)
         return None, dk.to(ctx.wn_dtype), None, None, None

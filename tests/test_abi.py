@@ -29,7 +29,7 @@ def test_version_and_strerror():
     lib = _lib.load()
     assert lib.proteus_version() >= 100
     assert lib.proteus_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert lib.proteus_strerror(code) not in (b"", b"unknown error code")
     assert lib.proteus_strerror(-99) == b"unknown error code"
 

@@ -101,6 +101,17 @@ def test_gradients_through_the_operators(gpu):
     _, cs, ss = pa.we_forward(coords.to(gpu), wn.to(gpu), mask.to(gpu))
     assert rel_l2(w.grad.cpu().numpy(), iso_reference(dO.cpu(), cs.cpu(), ss.cpu()).numpy()) <= REL_L2_TOL
 
+    # NaN / Inf in the padded positions of the coordinates reach neither the saved sums nor the gradient
+    dirty = coords.clone()
+    dirty[mask] = torch.tensor([float("nan"), float("inf"), -1e30])
+    w_d = wn.to(gpu).requires_grad_(True)
+    pa.wf_embedding(dirty.to(gpu), w_d, mask=mask.to(gpu)).backward(dO)
+    assert torch.isfinite(w_d.grad).all() and rel_l2(w_d.grad.cpu().numpy(), w.grad.cpu().numpy()) <= REL_L2_TOL
+    # a gradient asked of the coordinates only (there is none): backward returns nothing instead of failing
+    c_req = coords.to(gpu).requires_grad_(True)
+    pa.wf_embedding(c_req, wn.to(gpu), mask=mask.to(gpu)).backward(dO)
+    assert c_req.grad is None
+
     cb_dir = torch.randn(2, 300, 3, generator=g)
     cb_dir = cb_dir / cb_dir.norm(dim=-1, keepdim=True)
     cbm = (0.5 + torch.rand(48, generator=g)).to(gpu).requires_grad_(True)

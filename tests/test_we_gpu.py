@@ -129,6 +129,18 @@ def test_masks(gpu):
     sub = run_gpu(gpu, coords[0:1, keep], wn)
     for a, b in zip(got, sub):
         assert rel_l2(a[0][keep.numpy()], b[0]) < 1e-5
+    # what padded positions hold (NaN, Inf, huge) reaches nothing: padded rows stay exact zeros, valid rows keep their values
+    junk = torch.tensor([float("nan"), float("inf"), -float("inf"), 3e38, -1e30])
+    dirty = coords.clone()
+    dirty[mask] = junk[torch.randint(0, 5, (int(mask.sum()), 3), generator=g)]
+    for tuning in range(len(_lib.we_variants())):
+        bad = run_gpu(gpu, dirty, wn, mask, tuning=tuning)
+        for a, b in zip(bad, got):
+            assert np.isfinite(a).all(), f"variant {tuning}"
+            assert (a[mask.numpy()] == 0).all()
+            assert rel_l2(a, b) < 1e-5
+    no_sums = pa.we_forward(dirty.to(gpu), wn.to(gpu), mask.to(gpu), need_sums=False)[0].cpu().numpy()
+    assert np.isfinite(no_sums).all() and (no_sums[mask.numpy()] == 0).all() and rel_l2(no_sums, got[0]) < 1e-5
 
 
 def test_coincident_points_and_reference_sentinel(gpu):
