@@ -191,3 +191,48 @@ def geo_attn_autograd_torch(Q, K, V, coords, sigma, key_padding_mask=None, betas
     T = torch.where(row_any, T, torch.zeros_like(T))
     P = torch.softmax(T, dim=-1) * row_any.to(dtype)
     return torch.matmul(P, V)
+
+
+def geo_attn_scalar_grad_mass(Q, K, V, dO, coords, sigma, key_padding_mask=None, betas=None, min_rbf=0.0, max_rbf=1.0,
+                              dtype=torch.float64):
+    """Scale of the rounding error of d_sigma and d_beta: (mass_sigma [H], mass_beta [H] | None, and the same two
+    sums with their signs kept, which are the gradients themselves and pin the terms against torch.autograd).
+
+    Both gradients are sums over the pairs of P (dP - D) dT/d(sigma | beta), dP = dO . V, D = sum_j P dP, in which dP
+    and D largely cancel (exactly, for a query with one surviving pair).  A kernel whose P, dP or D carry a relative
+    error eps leaves about eps times
+        mass = sum_pairs P (|dP| + |D|) |dT/d(sigma | beta)|
+    however small the gradient itself comes out; tests hold the kernel to a fraction of this mass.  It is a bound on
+    magnitudes only; GPU tests take no gradient value from it (tests/test_oracle_attn.py checks the signed sums of the
+    same terms against autograd through geo_attn_autograd_torch).
+    Logits as in geo_attn_autograd_torch (old/old_scripts/attn/geometric_attn.py:193-201 with betas, README.md:40 without)."""
+    Q, K, V, dO = Q.to(dtype), K.to(dtype), V.to(dtype), dO.to(dtype)
+    coords, sigma = coords.to(dtype), sigma.to(dtype)
+    Z, H, N, d = Q.shape
+    mask = torch.zeros(Z, N, dtype=torch.bool) if key_padding_mask is None else key_padding_mask.bool()
+    S = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(d)
+    d2 = torch.sum((coords[:, :, None, :] - coords[:, None, :, :]) ** 2, dim=3)[:, None, :, :]
+    sg = sigma[None, :, None, None]
+    rbf = torch.exp(-d2 / (2 * sg ** 2))
+    drbf = rbf * d2 / sg ** 3                                   # d rbf / d sigma
+    am = (mask[:, None, :, None] | mask[:, None, None, :]).expand(Z, H, N, N)
+    if betas is None:
+        T = S * (1 + rbf)
+        w_sigma, w_beta = S * drbf, None
+    else:
+        am = am | (rbf < min_rbf) | (rbf > max_rbf)
+        bt = betas.to(dtype)[None, :, None, None]
+        rn = (2 * (rbf - min_rbf) / (max_rbf - min_rbf)) - 1
+        T = S + bt * rn * S.abs()
+        w_sigma, w_beta = bt * (2 / (max_rbf - min_rbf)) * drbf * S.abs(), rn * S.abs()
+    T = torch.where(am, torch.full_like(T, float("-inf")), T)
+    row_any = (~am).any(dim=-1, keepdim=True)
+    T = torch.where(row_any, T, torch.zeros_like(T))
+    P = torch.softmax(T, dim=-1) * row_any.to(dtype)
+    dP = torch.matmul(dO, V.transpose(2, 3))
+    D = (P * dP).sum(dim=-1, keepdim=True)
+    spread, signed = P * (dP.abs() + D.abs()), P * (dP - D)
+    mass_sigma, total_sigma = (spread * w_sigma.abs()).sum(dim=(0, 2, 3)), (signed * w_sigma).sum(dim=(0, 2, 3))
+    if w_beta is None:
+        return mass_sigma, None, total_sigma, None
+    return mass_sigma, (spread * w_beta.abs()).sum(dim=(0, 2, 3)), total_sigma, (signed * w_beta).sum(dim=(0, 2, 3))

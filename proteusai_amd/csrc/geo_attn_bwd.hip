@@ -396,6 +396,10 @@ void geo_attn_bwd_body(BwdSmem& sm, const int block_id,
             }
     }
     if (!OWN_Q) {
+        // A lane's sums hold the pairs of its own key only.  For an unusable own key they are worth nothing, and not
+        // even zero for sure: its scores are 0, so against a query with a very negative L its P can overflow (its dK
+        // and dV columns are overwritten with zeros above; here inf * 0 would leave a NaN).
+        if (!own_use) { sum_sigma = 0.f; sum_beta = 0.f; }
         for (int off = 32; off > 0; off >>= 1) {
             sum_sigma += __shfl_xor(sum_sigma, off);
             if (LEGACY) sum_beta += __shfl_xor(sum_beta, off);

@@ -116,6 +116,13 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
 }
 
+// c + the two bf16 values packed in w (v_dot2_f32_bf16 against ones).  The softmax row sum is taken over the
+// probabilities AS THE P.V PRODUCT SEES THEM (rounded to bf16), so O is a convex combination of V rows to fp32
+// rounding and D = rowsum(O dO) cancels against dP in the backward the way the exact quantities do.
+__device__ __forceinline__ float add_packed_bf16(const unsigned w, const float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), __builtin_bit_cast(bf16x2, 0x3f803f80u), c, false);
+}
+
 // a = h + m + l with h, m, l representable in bf16 (exact for any finite float whose pieces do not underflow)
 __device__ __forceinline__ void split3(float a, float& h, float& m, float& l) {
     h = (float)(__bf16)a;
@@ -234,11 +241,18 @@ void geo_attn_fwd_body(Smem& sm, const int block_id,
     const float oy = 0.5f * (cz[3 * q_first + 1] + cz[3 * q_last + 1]);
     const float oz = 0.5f * (cz[3 * q_first + 2] + cz[3 * q_last + 2]);
     const int q_mirror = (wave_first != 0x7fffffff) ? wave_first : q_first;
+    // With the reference's logits on the direct-distance path the rbf decides a pair mask, so it is evaluated
+    // exactly as the backward kernel evaluates it (raw coordinates, exp2(-d^2 cs2), same operation order): a pair is
+    // then in range in both or in neither.
+    constexpr bool RAW_DIST = LEGACY && DIST_VALU;
+    const float cs2 = 0.72134752044448170368f / (sg * sg);       // log2(e)/2 / sigma^2
     float qx[GA_QB], qy[GA_QB], qz[GA_QB], qn2[GA_QB];
+    float qrx[GA_QB], qry[GA_QB], qrz[GA_QB];
 #pragma unroll
     for (int b = 0; b < GA_QB; ++b) {
         const int qc = q_ok[b] ? q[b] : q_mirror;      // a padded lane mirrors a valid query: finite, in-range data
-        qx[b] = (cz[3 * qc] - ox) * cscale; qy[b] = (cz[3 * qc + 1] - oy) * cscale; qz[b] = (cz[3 * qc + 2] - oz) * cscale;
+        qrx[b] = cz[3 * qc]; qry[b] = cz[3 * qc + 1]; qrz[b] = cz[3 * qc + 2];
+        qx[b] = (qrx[b] - ox) * cscale; qy[b] = (qry[b] - oy) * cscale; qz[b] = (qrz[b] - oz) * cscale;
         qn2[b] = qx[b] * qx[b] + qy[b] * qy[b] + qz[b] * qz[b];
     }
     {
@@ -442,7 +456,14 @@ void geo_attn_fwd_body(Smem& sm, const int block_id,
             unsigned* dst = reinterpret_cast<unsigned*>(&tb.geo[gkey * GA_LDG + 6 * gcmp]);
             dst[0] = w0; dst[1] = w1; dst[2] = w2;
         } else if (gcmp == 0) {
-            tb.cx[gkey] = gx; tb.cy[gkey] = gy; tb.cz[gkey] = gz;
+            if (RAW_DIST) {
+                const bool gone = (mz && mg) || (loaded_j0 + gkey >= N);
+                tb.cx[gkey] = gone ? 0.f : __builtin_bit_cast(float, rx);
+                tb.cy[gkey] = gone ? 0.f : __builtin_bit_cast(float, ry);
+                tb.cz[gkey] = gone ? 0.f : __builtin_bit_cast(float, rz);
+            } else {
+                tb.cx[gkey] = gx; tb.cy[gkey] = gy; tb.cz[gkey] = gz;
+            }
         }
         if (tid < GA_BN) {
             tb.bias[tid] = kvalid ? 0.f : -INFINITY;
@@ -482,9 +503,17 @@ void geo_attn_fwd_body(Smem& sm, const int block_id,
                     const float kzs[4] = {kz.x, kz.y, kz.z, kz.w};
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        const float dx = qx[b] - kxs[v], dy = qy[b] - kys[v], dz = qz[b] - kzs[v];
-                        const float d2 = dx * dx + dy * dy + dz * dz;
-                        sacc[4 * g + v] = __builtin_fmaf(apply_rbf(sacc[4 * g + v], __builtin_amdgcn_exp2f(-d2)), log2e, mneg);
+                        float rbf;
+                        if (RAW_DIST) {
+                            const float dx = qrx[b] - kxs[v], dy = qry[b] - kys[v], dz = qrz[b] - kzs[v];
+                            const float d2 = __builtin_fmaf(dz, dz, __builtin_fmaf(dy, dy, dx * dx));
+                            rbf = __builtin_amdgcn_exp2f(-d2 * cs2);
+                        } else {
+                            const float dx = qx[b] - kxs[v], dy = qy[b] - kys[v], dz = qz[b] - kzs[v];
+                            const float d2 = dx * dx + dy * dy + dz * dz;
+                            rbf = __builtin_amdgcn_exp2f(-d2);
+                        }
+                        sacc[4 * g + v] = __builtin_fmaf(apply_rbf(sacc[4 * g + v], rbf), log2e, mneg);
                     }
                 }
             }
@@ -507,11 +536,10 @@ void geo_attn_fwd_body(Smem& sm, const int block_id,
                 // contraction slot e of this half-wave is key mt*32 + 16*t + 8*(e/4) + 4*half + (e%4)
                 float p[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    p[e] = __builtin_amdgcn_exp2f(sacc[8 * t + e]);
-                    lsum += p[e];
-                }
+                for (int e = 0; e < 8; ++e) p[e] = __builtin_amdgcn_exp2f(sacc[8 * t + e]);
                 pb[t] = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+                lsum = add_packed_bf16(pb[t].x, lsum); lsum = add_packed_bf16(pb[t].y, lsum);
+                lsum = add_packed_bf16(pb[t].z, lsum); lsum = add_packed_bf16(pb[t].w, lsum);
             }
         };
         exponentials();

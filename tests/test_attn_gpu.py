@@ -19,7 +19,11 @@ from proteusai_amd import _lib, synth
 pytestmark = pytest.mark.gpu
 
 MAX_ABS_TOL = 2e-2         # the stated parity bar for bf16 attention
-LSE_TOL = 1e-3             # the logsumexp never sees bf16 probabilities
+# The kernels sum the bf16-ROUNDED probabilities (the ones the P V product uses), so that the weights of O add up to
+# exactly one and rowsum(O dO) cancels against dP in the backward.  Each term is off by at most 2^-8 of itself (bf16
+# keeps 8 significant bits), hence so is the sum, and |logsumexp error| <= 2^-8 = 3.9e-3 (measured: up to 3.8e-3 for rows
+# that one key dominates, around 1e-3 for rows with many keys).
+LSE_TOL = 4.0e-3
 
 
 def make(seed, Z, H, N, qscale=1.0, maskfrac=0.0, tail=False):
@@ -357,7 +361,8 @@ def test_legacy_logits(gpu):
         assert np.abs(L[fin] - Lr[fin]).max() <= LSE_TOL
     # module: the reference's GeoAttention semantics (beta = exp(w), min_rbf default) are available on request
     torch.manual_seed(1)
-    mod = pa.GeoAttention(d_model=128, heads=2, min_rbf=0.001, legacy_logits=True).to(gpu)
+    mod = pa.GeoAttention(d_model=128, heads=2, legacy_logits=True).to(gpu)
+    assert mod.min_rbf == 0.001 and pa.GeoAttention(d_model=128, heads=2).min_rbf == 0.0      # old/old_scripts/encoder.py:57
     x = torch.randn(1, 70, 128)
     with torch.no_grad():
         y = mod(x.to(gpu), x.to(gpu), x.to(gpu), coords[:1, :70].to(gpu))

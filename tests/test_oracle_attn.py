@@ -200,3 +200,13 @@ def test_per_query_sigma_and_beta_split_the_per_head_gradients():
         assert (s_rows.grad[mask[:, None, :].expand(Z, H, N)] == 0).all()          # a padded query contributes nothing
         if betas is not None:
             assert torch.allclose(b_rows.grad.sum(dim=(0, 2)), b_head.grad, rtol=1e-10, atol=1e-12)
+        # the pair-level error scale of the per-head scalars: its terms, signs kept, ARE the gradients (autograd's), and
+        # it bounds what survives the cancellation inside a query and between the queries
+        m_s, m_b, t_s, t_b = torch_oracle.geo_attn_scalar_grad_mass(Q, K, V, dO, coords, s_head.detach(), mask, betas, lo, hi)
+        assert torch.allclose(t_s, s_head.grad, rtol=1e-9, atol=1e-12)
+        assert (m_s >= s_rows.grad.abs().sum(dim=(0, 2)) * (1 - 1e-12)).all() and (m_s > 0).all()
+        if betas is not None:
+            assert torch.allclose(t_b, b_head.grad, rtol=1e-9, atol=1e-12)
+            assert (m_b >= b_rows.grad.abs().sum(dim=(0, 2)) * (1 - 1e-12)).all()
+        else:
+            assert m_b is None and t_b is None

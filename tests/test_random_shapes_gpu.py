@@ -50,7 +50,7 @@ def test_wavefunction_embeddings(gpu, case):
         assert rel_l2(g, r) <= 1e-4, f"{what} aniso {name}: {rel_l2(g, r):.3e}"
 
 
-@pytest.mark.parametrize("case", range(12))
+@pytest.mark.parametrize("case", range(160))
 def test_attention_forward_and_backward(gpu, case):
     rng = np.random.default_rng(2000 + case)
     Z, H, N = int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.integers(1, 400))
@@ -104,13 +104,23 @@ def test_attention_forward_and_backward(gpu, case):
             assert rel_l2(gg, rr.numpy()) <= 1e-2, f"{what} {name}: {rel_l2(gg, rr.numpy()):.3e}"
         else:
             assert np.abs(gg).max() <= 1e-6, f"{what} {name}"
-    # Per-head scalars: sums of terms of both signs.  Always within 1 % of the absolute mass of the per-query
-    # contributions; within 1 % of the value itself where at least a quarter of that mass survives the cancellation.
-    for gg, rows, name in [(s.grad, rs.grad, "d_sigma")] + ([(bt.grad, rb.grad, "d_beta")] if legacy else []):
+    # Per-head scalars: sums over pairs of P (dP - D) dT/d(scalar), terms of both signs that cancel inside a query and
+    # between queries.  Always within 2^-9 of what went into the sum before any cancellation (the oracle's pair mass: no
+    # case and no term is left out; the forward's bf16 probabilities differ from the backward's fp32 ones by up to 2^-8
+    # per pair, measured over this sweep: <= 4.5e-4); within 1 % of the value itself where it keeps a quarter of that mass.
+    mass_s, mass_b, _, _ = torch_oracle.geo_attn_scalar_grad_mass(Q, K, V, dO, coords, sigma, mask, betas, lo, hi)
+    for gg, rows, pair_mass, name in [(s.grad, rs.grad, mass_s, "d_sigma")] + ([(bt.grad, rb.grad, mass_b, "d_beta")] if legacy else []):
         gg = gg.double().cpu()
-        total, mass = rows.sum(dim=(0, 2)), rows.abs().sum(dim=(0, 2))
+        total = rows.sum(dim=(0, 2))
         assert torch.isfinite(gg).all(), f"{what} {name}"
         err = (gg - total).abs()
-        assert (err <= 1e-2 * mass + 1e-9).all(), f"{what} {name}: error / mass {(err / mass.clamp_min(1e-300)).max():.3e}"
-        if (total.abs() >= 0.25 * mass).all() and total.norm() > 1e-9:
+        assert (err <= 2.0 ** -9 * pair_mass + 1e-30).all(), \
+            f"{what} {name}: error / pair mass {(err / pair_mass.clamp_min(1e-300)).max():.3e}"
+        if (total.abs() >= 0.25 * pair_mass).all() and total.norm() > 1e-9:
             assert rel_l2(gg.numpy(), total.numpy()) <= 1e-2, f"{what} {name}: {rel_l2(gg.numpy(), total.numpy()):.3e}"
+    if not legacy:
+        # the software-pipelined forward is the default only for large grids: force it on the same inputs
+        O5 = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), tuning=5).cpu().double()
+        assert torch.isfinite(O5).all(), what
+        assert (O5 - Oref.detach()).abs().max() <= 2e-2, f"{what}: pipelined O {(O5 - Oref.detach()).abs().max():.3e}"
+        assert (O5[mask[:, None, :].expand(-1, H, -1)] == 0).all(), what
