@@ -1,16 +1,21 @@
 """Headline benchmark: Wavefunction Embedding forward at B=1, N=16384, d_model=512
-(BASELINE.json configs[1]) on one MI355X, with the geometric attention forward at
-N=16384, H=8, d=64 measured beside it, roofline fractions for both kernels and
-the CPU PyTorch path timed on the host cores as a baseline.
+(BASELINE.json configs[1]) on one MI355X.  Beside it, one timed leg per other configuration
+(configs[0] WE N=512; configs[2] padded attention B=4 N=4096; configs[3] encoder forward;
+configs[4] WE N=65536 and attention N=16384), roofline fractions for every kernel and the
+CPU PyTorch path timed on the host cores as a baseline for each.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-attn]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--legs a,b,...] [--no-cpu] [--full-cpu]
 
 Prints ONE JSON line.  A "step" is one WE forward over the whole batch, inputs
 and outputs resident in HBM, outputs pre-allocated.
+
+Counter-derived fields (traffic, mfma_util, valu_insts_per_unit) are read from the rocprofv3
+summaries under profiles/ (lines of the form "name = number"); each carries a "source" key.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,25 +29,70 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0      # dense bf16 matrix
 PEAK_HBM_GBS = 8000.0               # HBM3E
 H100_REFERENCE_GPW = 6.87194767e10 / 0.386 / 1e9   # README.md:34: 386 ms at this exact shape on an H100
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), bytes
-# WE: FETCH_SIZE 4370.5 KiB x 2.0 (calibration factor of that counter) + WRITE_SIZE 82271.9 KiB x 1.0
-WE_TRAFFIC_BYTES = int((4370.5 * 2.0 + 82271.9) * 1024)
-# attention: FETCH_SIZE 43028.5 KiB x 2.0 (both distance-path bodies of the one launch) + WRITE_SIZE 33792.0 KiB x 1.0
-ATTN_TRAFFIC_BYTES = int((43028.5 * 2.0 + 33792.0) * 1024)
+LEGS = ("we_lean", "we_bwd", "aniso", "cfg1", "cfg3", "cfg5_we", "attn", "attn_bwd", "encoder")
+PROFILE_WE = "profiles/we_fwd_N16384_K256__counters.txt"
+PROFILE_ATTN = "profiles/geo_attn_fwd_N16384_H8_d64__counters.txt"
+PROFILE_ATTN_BWD = "profiles/geo_attn_bwd_N16384_H8_d64__counters.txt"
 
 
-def median(xs):
-    xs = sorted(xs)
-    return xs[len(xs) // 2]
+def read_profile(rel):
+    """{name: float} from the 'name = number' lines of a summary under profiles/ ({} if the file is absent)."""
+    vals = {}
+    try:
+        with open(os.path.join(ROOT, rel)) as f:
+            for line in f:
+                m = re.match(r"^\s*([A-Za-z_][A-Za-z0-9_.]*)\s*=\s*([-+0-9.eE]+)\s*(#.*)?$", line)
+                if m:
+                    vals[m.group(1)] = float(m.group(2))
+    except OSError:
+        pass
+    return vals
+
+
+def traffic_from(rel):
+    """HBM bytes per launch from FETCH_SIZE / WRITE_SIZE (KiB per dispatch) and the copy-kernel calibration factors."""
+    p = read_profile(rel)
+    need = ("FETCH_SIZE_KiB", "FETCH_SIZE_scale", "WRITE_SIZE_KiB", "WRITE_SIZE_scale")
+    if not all(k in p for k in need):
+        return None, None
+    return int((p["FETCH_SIZE_KiB"] * p["FETCH_SIZE_scale"] + p["WRITE_SIZE_KiB"] * p["WRITE_SIZE_scale"]) * 1024), rel
 
 
 def settle(torch, fn, min_ms=60.0):
     """Run fn untimed for at least min_ms: while a leg's inputs are made on the host the GPU idles and drops its
     clocks, and the first ~25 ms of work afterwards run below the sustained rate."""
     t0 = time.perf_counter()
-    while (time.perf_counter() - t0) * 1e3 < min_ms:
+    while True:
         fn()
         torch.cuda.synchronize()
+        if (time.perf_counter() - t0) * 1e3 >= min_ms:
+            break
+
+
+def time_launches(torch, fn, n, min_settle_ms=60.0):
+    """(mean ms, median ms) of n launches of fn, each bracketed by events on torch's current stream (the stream every
+    leg passes to the library)."""
+    settle(torch, fn, min_settle_ms)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for e0, e1 in ev:
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = sorted(e0.elapsed_time(e1) for e0, e1 in ev)
+    return sum(ms) / n, ms[n // 2]
+
+
+def cpu_timed(fn, budget_s, max_runs):
+    """Median wall time of up to max_runs runs of fn, stopping once budget_s is spent (always at least one run)."""
+    times, spent = [], 0.0
+    while len(times) < max_runs and (not times or spent + times[-1] <= budget_s):
+        t = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t)
+        spent += times[-1]
+    times.sort()
+    return times[len(times) // 2], len(times)
 
 
 def probe_rates(lib, torch, dev):
@@ -70,11 +120,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-attn", action="store_true", help="skip the geometric attention leg")
-    ap.add_argument("--no-aniso", action="store_true", help="skip the anisotropic WE leg")
-    ap.add_argument("--no-encoder", action="store_true", help="skip the encoder-forward leg (BASELINE.json configs[3])")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--legs", default="all", help="comma-separated legs beside the headline one: " + ",".join(LEGS) + ", all, none")
+    ap.add_argument("--no-cpu", action="store_true", help="skip every CPU baseline")
+    ap.add_argument("--full-cpu", action="store_true",
+                    help="run the CPU path of the headline shape (and of the N=16384 attention) in full, once, instead of on a sample of rows")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the headline CPU baseline sample")
     ap.add_argument("--we-tuning", type=int, default=0)
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch a 256 MiB device copy, so a rocprofv3 --pmc run of this command holds a kernel of known traffic")
@@ -83,6 +133,11 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (observer rows and (batch, head) pairs are "
               "independent, so the work shards without any exchange); "
               "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    legs = set(LEGS) if args.legs == "all" else set() if args.legs == "none" else set(args.legs.split(","))
+    unknown = legs - set(LEGS)
+    if unknown:
+        print(f"unknown legs: {sorted(unknown)}", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -93,6 +148,18 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    threads = torch.get_num_threads()
+    if not args.no_cpu:
+        from oracle import torch_oracle
+
+    def we_forward_into(c, w, m, out, cs, ss, tuning=0):
+        Zc, Nc, _ = c.shape
+        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(), None if m is None else m.data_ptr(), out.data_ptr(),
+                                None if cs is None else cs.data_ptr(), None if ss is None else ss.data_ptr(),
+                                Zc, Nc, w.numel(), tuning, stream)
+        if rc != 0:
+            _lib.check(rc, "proteus_we_fwd")
 
     # ---------------- WE forward, B=1, N=16384, d_model=512, compacted random-walk chain ----------------
     Z, N, d_model = 1, 16384, 512
@@ -102,13 +169,9 @@ def main():
     out = torch.empty(Z, N, 2 * K, device=dev)
     cs = torch.empty(Z, N, K, device=dev)
     ss = torch.empty(Z, N, K, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
 
     def we_step():
-        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(), None, out.data_ptr(), cs.data_ptr(),
-                                ss.data_ptr(), Z, N, K, args.we_tuning, stream)
-        if rc != 0:
-            _lib.check(rc, "proteus_we_fwd")
+        we_forward_into(c, w, None, out, cs, ss, args.we_tuning)
 
     for _ in range(args.warmup):
         we_step()
@@ -131,11 +194,14 @@ def main():
     rates = probe_rates(lib, torch, dev)
     # per unit: the phase product (scalar operand), v_sin, v_cos, two v_fmac and two v_add on vector operands
     r_trans = (rates["sin"] + rates["cos"]) / 2
-    t_model_ms = W * (1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / rates["add_v"] + 2.0 / r_trans) * 1e3
+    per_unit_s = 1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / rates["add_v"] + 2.0 / r_trans
+    t_model_ms = W * per_unit_s * 1e3
     achieved_tflops = 9.0 * W / (avg_kernel_ms * 1e-3) / 1e12   # 9 flop per unit, FMA counted as 2
+    we_traffic, we_traffic_src = traffic_from(PROFILE_WE)
     roofline = {
         "kernel": "we_fwd_kernel", "bound": "valu", "achieved": achieved_tflops, "peak": PEAK_FP32_VECTOR_TFLOPS,
-        "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_FP32_VECTOR_TFLOPS, "traffic": WE_TRAFFIC_BYTES,
+        "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_FP32_VECTOR_TFLOPS,
+        "traffic": we_traffic, "traffic_source": we_traffic_src,
         "kernel_ms": avg_kernel_ms,
         "issue_model": {
             "lane_ops_per_unit": {"mul_scalar_operand": 1, "fmac_vector_operands": 2, "add_vector_operands": 2,
@@ -145,6 +211,12 @@ def main():
             "model_ms": t_model_ms, "frac": t_model_ms / avg_kernel_ms,
         },
     }
+    pw = read_profile(PROFILE_WE)
+    if "valu_insts_per_unit" in pw:
+        roofline["valu_insts_per_unit"] = {
+            "value": pw["valu_insts_per_unit"], "add_f32": pw.get("add_f32_per_unit"), "mul_f32": pw.get("mul_f32_per_unit"),
+            "fma_f32": pw.get("fma_f32_per_unit"), "trans_f32": pw.get("trans_f32_per_unit"),
+            "valu_active_frac": pw.get("valu_active_frac"), "source": PROFILE_WE}
 
     result = {
         "metric": "we_fwd_gpair_wavenumber_per_s", "value": value, "unit": "Gpair*wavenumber/s",
@@ -159,63 +231,46 @@ def main():
         "roofline": roofline,
     }
 
+    def we_model_frac(units, ms):
+        return units * per_unit_s * 1e3 / ms
+
     # ---------------- the same forward without the cos/sin sums (inference: nothing kept for a backward) ----------
-    def we_lean_step():
-        rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(), None, out.data_ptr(), None, None,
-                                Z, N, K, args.we_tuning, stream)
-        if rc != 0:
-            _lib.check(rc, "proteus_we_fwd")
-    for _ in range(2):
-        we_lean_step()
-    torch.cuda.synchronize()
-    n_lean = max(5, args.steps // 2)
-    lev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_lean)]
-    for e0, e1 in lev:
-        e0.record()
-        we_lean_step()
-        e1.record()
-    torch.cuda.synchronize()
-    lean_ms = sum(e0.elapsed_time(e1) for e0, e1 in lev) / n_lean
-    # per unit: the phase product, v_sin, v_cos and two v_fmac (the two v_add of the plain sums are gone)
-    lean_model_ms = W * (1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / r_trans) * 1e3
-    result["we_fwd_without_sums"] = {
-        "workload": "the headline shape with cos_sums = sin_sums = NULL (embedding only; not the headline metric, "
-                    "whose forward also returns the sums as the reference's does)",
-        "ms": lean_ms, "gpair_wavenumber_per_s": W / (lean_ms * 1e-3) / 1e9, "dtype": "f32",
-        "issue_model": {"model_ms": lean_model_ms, "frac": lean_model_ms / lean_ms},
-    }
+    if "we_lean" in legs:
+        lean_ms, _ = time_launches(torch, lambda: we_forward_into(c, w, None, out, None, None, args.we_tuning), max(5, args.steps // 2), 0.0)
+        # per unit: the phase product, v_sin, v_cos and two v_fmac (the two v_add of the plain sums are gone)
+        lean_model_ms = W * (1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / r_trans) * 1e3
+        result["we_fwd_without_sums"] = {
+            "workload": "the headline shape with cos_sums = sin_sums = NULL (embedding only; not the headline metric, "
+                        "whose forward also returns the sums as the reference's does)",
+            "ms": lean_ms, "gpair_wavenumber_per_s": W / (lean_ms * 1e-3) / 1e9, "dtype": "f32",
+            "issue_model": {"model_ms": lean_model_ms, "frac": lean_model_ms / lean_ms},
+        }
 
     # ---------------- WE backward (the reduction of dO against the sums), same shape: HBM-bound ----------------
-    dO = torch.randn(Z, N, 2 * K, device=dev)
-    dk = torch.empty(K, device=dev)
-    ws_bytes = lib.proteus_we_bwd_workspace_bytes(Z, N, K)
-    ws = torch.empty(ws_bytes // 4, device=dev)
+    if "we_bwd" in legs:
+        dO = torch.randn(Z, N, 2 * K, device=dev)
+        dk = torch.empty(K, device=dev)
+        ws_bytes = lib.proteus_we_bwd_workspace_bytes(Z, N, K)
+        ws = torch.empty(ws_bytes // 4, device=dev)
 
-    def we_bwd_step():
-        rc = lib.proteus_we_bwd(dO.data_ptr(), cs.data_ptr(), ss.data_ptr(), dk.data_ptr(), ws.data_ptr(), ws_bytes,
-                                Z, N, K, stream)
-        if rc != 0:
-            _lib.check(rc, "proteus_we_bwd")
-    settle(torch, we_bwd_step)
-    bev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
-    for e0, e1 in bev:
-        e0.record()
-        we_bwd_step()
-        e1.record()
-    torch.cuda.synchronize()
-    b_ms = sorted(e0.elapsed_time(e1) for e0, e1 in bev)[len(bev) // 2]
-    b_bytes = 16.0 * Z * N * K                       # dO (8) + cos_sums (4) + sin_sums (4) per (token, wavenumber)
-    result["we_bwd"] = {
-        "workload": "WE backward for the wavenumbers, dO [1,16384,512] against the saved sums, two launches",
-        "ms": b_ms, "dtype": "f32",
-        "roofline": {"kernel": "we_bwd_partial_kernel + we_bwd_final_kernel", "bound": "hbm",
-                     "achieved": b_bytes / (b_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": b_bytes / (b_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None},
-    }
-    del dO, ws
+        def we_bwd_step():
+            rc = lib.proteus_we_bwd(dO.data_ptr(), cs.data_ptr(), ss.data_ptr(), dk.data_ptr(), ws.data_ptr(), ws_bytes,
+                                    Z, N, K, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_we_bwd")
+        _, b_ms = time_launches(torch, we_bwd_step, 20)
+        b_bytes = 16.0 * Z * N * K                       # dO (8) + cos_sums (4) + sin_sums (4) per (token, wavenumber)
+        result["we_bwd"] = {
+            "workload": "WE backward for the wavenumbers, dO [1,16384,512] against the saved sums, two launches",
+            "ms": b_ms, "dtype": "f32",
+            "roofline": {"kernel": "we_bwd_partial_kernel + we_bwd_final_kernel", "bound": "hbm",
+                         "achieved": b_bytes / (b_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": b_bytes / (b_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None},
+        }
+        del dO, ws
 
     # ---------------- anisotropic (C-beta scaled) WE forward, same shape and chain ----------------
-    if not args.no_aniso:
+    if "aniso" in legs:
         g = torch.Generator().manual_seed(2)
         cbv = torch.randn(Z, N, 3, generator=g)
         cbv = (cbv / cbv.norm(dim=-1, keepdim=True)).to(dev).contiguous()
@@ -227,17 +282,7 @@ def main():
                                           ao[0].data_ptr(), ao[1].data_ptr(), ao[2].data_ptr(), Z, N, K, 0, stream)
             if rc != 0:
                 _lib.check(rc, "proteus_we_aniso_fwd")
-        for _ in range(2):
-            aniso_step()
-        torch.cuda.synchronize()
-        n_it = max(5, args.steps // 2)
-        xev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_it)]
-        for e0, e1 in xev:
-            e0.record()
-            aniso_step()
-            e1.record()
-        torch.cuda.synchronize()
-        x_ms = sum(e0.elapsed_time(e1) for e0, e1 in xev) / n_it
+        x_ms, _ = time_launches(torch, aniso_step, max(5, args.steps // 2), 0.0)
         # per unit: 2 scalar-operand phase ops, v_fract, 4 v_fmac + 2 v_add on vector operands, v_sin, v_cos
         x_model_ms = W * (2.0 / rates["mul_s"] + 1.0 / rates["fract"] + 4.0 / rates["fmac_v"] + 2.0 / rates["add_v"]
                           + 2.0 / r_trans) * 1e3
@@ -248,78 +293,164 @@ def main():
                                                   "add_vector_operands": 2, "transcendental": 2},
                             "model_ms": x_model_ms, "frac": x_model_ms / x_ms},
         }
+        del ao
+
+    # ---------------- configs[0]: WE forward B=1, N=512 (the reference's CPU-runnable case) ----------------
+    if "cfg1" in legs:
+        c1, _ = synth.we_inputs(512, seed=1, batch=1, d_model=d_model, compact=False)
+        c1d = c1.to(dev).contiguous()
+        o1, cs1, ss1 = (torch.empty(1, 512, n, device=dev) for n in (2 * K, K, K))
+        _, ms1 = time_launches(torch, lambda: we_forward_into(c1d, w, None, o1, cs1, ss1), 200)
+        W1 = 512.0 * 512 * K
+        leg = {"workload": "WE forward B=1 N=512 d_model=512, random-walk chain, no mask (BASELINE.json configs[0]); "
+                           "8 observer blocks of 64 rows x 4 wavenumber slices: 32 workgroups on 256 CUs, a launch-latency-sized kernel",
+               "ms": ms1, "gpair_wavenumber_per_s": W1 / (ms1 * 1e-3) / 1e9, "dtype": "f32",
+               "roofline": {"kernel": "we_fwd_kernel", "bound": "valu", "achieved": 9.0 * W1 / (ms1 * 1e-3) / 1e12,
+                            "peak": PEAK_FP32_VECTOR_TFLOPS, "unit": "TFLOP/s",
+                            "frac": 9.0 * W1 / (ms1 * 1e-3) / 1e12 / PEAK_FP32_VECTOR_TFLOPS,
+                            "issue_model_frac": we_model_frac(W1, ms1)}}
+        if not args.no_cpu:
+            dt, runs = cpu_timed(lambda: torch_oracle.we_torch(c1, wn), 10.0, 5)
+            leg["cpu_baseline"] = {"value": W1 / dt / 1e9, "unit": "Gpair*wavenumber/s", "cores": threads, "kind": "port",
+                                   "sample": f"the full workload, median of {runs} runs, tiled CPU PyTorch fp32, {dt * 1e3:.1f} ms"}
+        result["cfg1_we_n512"] = leg
+
+    # ---------------- configs[4], WE half: B=1, N=65536, same compacted-chain generator ----------------
+    if "cfg5_we" in legs:
+        c5, _ = synth.we_inputs(65536, seed=5, compact=True)
+        c5d = c5.to(dev).contiguous()
+        o5, cs5, ss5 = (torch.empty(1, 65536, n, device=dev) for n in (2 * K, K, K))
+        ms5, _ = time_launches(torch, lambda: we_forward_into(c5d, w, None, o5, cs5, ss5), 3, 0.0)
+        W5 = 65536.0 * 65536 * K
+        leg = {"workload": "WE forward B=1 N=65536 d_model=512, compacted random-walk chain, no mask (BASELINE.json configs[4])",
+               "ms": ms5, "gpair_wavenumber_per_s": W5 / (ms5 * 1e-3) / 1e9, "dtype": "f32",
+               "roofline": {"kernel": "we_fwd_kernel", "bound": "valu", "achieved": 9.0 * W5 / (ms5 * 1e-3) / 1e12,
+                            "peak": PEAK_FP32_VECTOR_TFLOPS, "unit": "TFLOP/s",
+                            "frac": 9.0 * W5 / (ms5 * 1e-3) / 1e12 / PEAK_FP32_VECTOR_TFLOPS,
+                            "issue_model_frac": we_model_frac(W5, ms5)}}
+        if not args.no_cpu:
+            sel = torch.linspace(0, 65535, 256).long().tolist()
+            t = time.perf_counter()
+            torch_oracle.we_torch(c5, wn, rows=sel)
+            dt = time.perf_counter() - t
+            leg["cpu_baseline"] = {"value": 256 * 65536.0 * K / dt / 1e9, "unit": "Gpair*wavenumber/s", "cores": threads,
+                                   "kind": "port", "extrapolated": True,
+                                   "sample": f"256 of 65536 observer rows (all 65536 sources each), tiled CPU PyTorch fp32, {dt:.1f} s; "
+                                             f"the full workload at this rate: {dt * 256:.0f} s"}
+        result["cfg5_we_n65536"] = leg
+        del o5, cs5, ss5, c5d
+
+    def attn_forward_into(q, k, v, cd, sg, m, O, L):
+        Za, Ha, Na, da = q.shape
+        rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), cd.data_ptr(), sg.data_ptr(),
+                                      None if m is None else m.data_ptr(), O.data_ptr(), L.data_ptr(), Za, Ha, Na, da, 0, stream)
+        if rc != 0:
+            _lib.check(rc, "proteus_geo_attn_fwd")
+
+    # ---------------- configs[2]: geometric attention B=4, N=4096, H=8, d=64, lengths in [2048, 4096] ----------------
+    if "cfg3" in legs:
+        Q3, K3, V3, c3, sg3, m3 = synth.attn_inputs(4, 8, 4096, 64, seed=3, min_len=2048)
+        q3, k3, v3, c3d, s3d, m3d = (t.to(dev) for t in (Q3, K3, V3, c3, sg3, m3))
+        O3 = torch.empty(4, 8, 4096, 64, device=dev)
+        L3 = torch.empty(4, 8, 4096, device=dev)
+        _, ms3 = time_launches(torch, lambda: attn_forward_into(q3, k3, v3, c3d, s3d, m3d, O3, L3), 50)
+        lens = (~m3).sum(dim=1).double()
+        useful = 4.0 * 8 * 64 * float((lens * lens).sum())
+        dense = 4.0 * 4 * 8 * 64 * 4096 * 4096
+        leg = {"workload": "geometric attention forward B=4 H=8 N=4096 d_head=64 bf16, random-walk chains, sigma 3-25 A, "
+                           "valid lengths uniform in [2048, 4096], the rest padded (BASELINE.json configs[2])",
+               "ms": ms3, "lengths": [int(x) for x in lens], "dtype": "bf16",
+               "tflops_useful": useful / (ms3 * 1e-3) / 1e12, "tflops_dense_equivalent": dense / (ms3 * 1e-3) / 1e12,
+               "roofline": {"kernel": "geo_attn_fwd_pipe_kernel", "bound": "mfma", "achieved": useful / (ms3 * 1e-3) / 1e12,
+                            "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
+                            "frac": useful / (ms3 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                            "flop": "4 H d sum_b L_b^2 (pairs of valid tokens only)"}}
+        if not args.no_cpu:
+            dt, runs = cpu_timed(lambda: torch_oracle.geo_attn_torch(Q3, K3, V3, c3, sg3, m3), 20.0, 3)
+            leg["cpu_baseline"] = {"value": dense / dt / 1e12, "unit": "TFLOP/s (dense-equivalent: the CPU path computes every pair and masks)",
+                                   "cores": threads, "kind": "port",
+                                   "sample": f"the full workload, median of {runs} run(s), dense CPU PyTorch fp32 on the bf16-rounded inputs, {dt:.1f} s"}
+        result["cfg3_attn_b4_n4096_padded"] = leg
+        del q3, k3, v3, O3, L3
 
     # ---------------- geometric attention forward, N=16384, H=8, d=64 (configs[4]) ----------------
-    if not args.no_attn:
+    if "attn" in legs or "attn_bwd" in legs:
         wc, _ = synth.we_inputs(65536, seed=5, compact=True)
         Q, Kt, V, ac, sigma, _ = synth.attn_inputs(1, 8, 16384, 64, seed=5, coords=wc[:, :16384].contiguous())
         q, k, v, acd, sg = Q.to(dev), Kt.to(dev), V.to(dev), ac.to(dev), sigma.to(dev)
         O = torch.empty(1, 8, 16384, 64, device=dev)
         L = torch.empty(1, 8, 16384, device=dev)
-
-        def attn_step():
-            rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), acd.data_ptr(), sg.data_ptr(), None,
-                                          O.data_ptr(), L.data_ptr(), 1, 8, 16384, 64, 0, stream)
-            if rc != 0:
-                _lib.check(rc, "proteus_geo_attn_fwd")
-        settle(torch, attn_step)
-        n_it = max(10, args.steps)
-        aev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_it)]
-        for e0, e1 in aev:
-            e0.record()
-            attn_step()
-            e1.record()
-        torch.cuda.synchronize()
-        a_ms = sum(e0.elapsed_time(e1) for e0, e1 in aev) / n_it
+        a_ms, _ = time_launches(torch, lambda: attn_forward_into(q, k, v, acd, sg, None, O, L), max(10, args.steps))
         flops = 4.0 * 8 * 64 * 16384 * 16384
         a_tflops = flops / (a_ms * 1e-3) / 1e12
-        result["geo_attn"] = {
+        a_traffic, a_traffic_src = traffic_from(PROFILE_ATTN)
+        leg = {
             "workload": "geometric attention forward Z=1 H=8 N=16384 d_head=64 bf16, compacted chain, sigma 3-25 A (BASELINE.json configs[4])",
             "ms": a_ms, "tflops": a_tflops, "dtype": "bf16",
-            "roofline": {"kernel": "geo_attn_fwd_kernel", "bound": "mfma", "achieved": a_tflops, "peak": PEAK_BF16_MFMA_TFLOPS,
-                         "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES},
+            "roofline": {"kernel": "geo_attn_fwd_pipe_kernel", "bound": "mfma", "achieved": a_tflops, "peak": PEAK_BF16_MFMA_TFLOPS,
+                         "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS,
+                         "traffic": a_traffic, "traffic_source": a_traffic_src},
         }
+        pa_ = read_profile(PROFILE_ATTN)
+        if "mfma_util" in pa_:
+            leg["roofline"]["mfma_util"] = {"value": pa_["mfma_util"], "mfma_flop_counted": pa_.get("mfma_flop"),
+                                            "lds_wait_frac": pa_.get("lds_wait_frac"), "source": PROFILE_ATTN}
+        if not args.no_cpu and "attn" in legs:
+            rows = None if args.full_cpu else torch.linspace(0, 16383, 1024).long().tolist()
+            t = time.perf_counter()
+            torch_oracle.geo_attn_torch(Q, Kt, V, ac, sigma, None, rows=rows)
+            dt = time.perf_counter() - t
+            n_rows = 16384 if rows is None else len(rows)
+            leg["cpu_baseline"] = {"value": flops * n_rows / 16384 / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                                   "extrapolated": rows is not None,
+                                   "sample": f"{n_rows} of 16384 query rows of every head (all 16384 keys each), dense CPU PyTorch fp32, {dt:.1f} s"}
+        result["geo_attn"] = leg
 
         # ---- backward of the same shape (dQ, dK, dV, d sigma from the forward's O and L) ----
-        gq = torch.Generator().manual_seed(5)
-        dOb = (torch.randn(1, 8, 16384, 64, generator=gq) / 8).bfloat16().to(dev)
-        Dv = (O * dOb.float()).sum(-1).contiguous()
-        dQ_, dK_, dV_ = (torch.empty(1, 8, 16384, 64, device=dev) for _ in range(3))
-        dsg = torch.zeros(8, device=dev)
+        if "attn_bwd" in legs:
+            gq = torch.Generator().manual_seed(5)
+            dOb = (torch.randn(1, 8, 16384, 64, generator=gq) / 8).bfloat16().to(dev)
+            Dv = (O * dOb.float()).sum(-1).contiguous()
+            dQ_, dK_, dV_ = (torch.empty(1, 8, 16384, 64, device=dev) for _ in range(3))
+            dsg = torch.zeros(8, device=dev)
 
-        def bwd_step():
-            rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dOb.data_ptr(), acd.data_ptr(), sg.data_ptr(),
-                                          None, None, L.data_ptr(), Dv.data_ptr(), dQ_.data_ptr(), dK_.data_ptr(), dV_.data_ptr(),
-                                          dsg.data_ptr(), None, 1, 8, 16384, 64, 0.0, 1.0, stream)
-            if rc != 0:
-                _lib.check(rc, "proteus_geo_attn_bwd")
-        settle(torch, bwd_step)
-        bev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(5)]
-        for e0, e1 in bev:
-            e0.record()
-            bwd_step()
-            e1.record()
-        torch.cuda.synchronize()
-        b_ms = sum(e0.elapsed_time(e1) for e0, e1 in bev) / len(bev)
-        result["geo_attn_bwd"] = {
-            "workload": "geometric attention backward, same shape: dQ, dK, dV, d_sigma (two passes in one launch, S and dP recomputed in each)",
-            "ms": b_ms, "tflops_5_products": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12,
-            "tflops_issued_7_products": 14.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12, "dtype": "bf16",
-        }
+            def bwd_step():
+                rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dOb.data_ptr(), acd.data_ptr(), sg.data_ptr(),
+                                              None, None, L.data_ptr(), Dv.data_ptr(), dQ_.data_ptr(), dK_.data_ptr(), dV_.data_ptr(),
+                                              dsg.data_ptr(), None, 1, 8, 16384, 64, 0.0, 1.0, stream)
+                if rc != 0:
+                    _lib.check(rc, "proteus_geo_attn_bwd")
+            b_ms, _ = time_launches(torch, bwd_step, 5)
+            b_traffic, b_traffic_src = traffic_from(PROFILE_ATTN_BWD)
+            result["geo_attn_bwd"] = {
+                "workload": "geometric attention backward, same shape: dQ, dK, dV, d_sigma (two passes in one launch, S and dP recomputed in each)",
+                "ms": b_ms, "tflops_5_products": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12,
+                "tflops_issued_7_products": 14.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12, "dtype": "bf16",
+                "roofline": {"kernel": "geo_attn_bwd_kernel", "bound": "mfma",
+                             "achieved": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
+                             "unit": "TFLOP/s", "frac": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                             "traffic": b_traffic, "traffic_source": b_traffic_src},
+            }
+            del dOb, Dv, dQ_, dK_, dV_
+        del q, k, v, O, L
 
     # ---------------- encoder forward, B=8, N=1024, 4 layers, bf16 weights, fp32 WE (configs[3]) ----------------
-    if not args.no_encoder:
+    if "encoder" in legs:
         import proteusai_amd as pa
         torch.manual_seed(4)
-        model = pa.ProteusEncoder().eval().to(dev)
+        model = pa.ProteusEncoder().eval()
+        state = {k_: v_.clone() for k_, v_ in model.state_dict().items()}
+        min_spread = model.layers[0].attn.min_spread
+        model.to(dev)
         model.aa_embedding.to(torch.bfloat16)
         model.layers.to(torch.bfloat16)
         model.head.to(torch.bfloat16)
         g = torch.Generator().manual_seed(4)
-        ecoords = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)]).to(dev)
-        etokens = torch.randint(0, 33, (8, 1024), generator=g).to(dev)
+        ecoords_h = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)])
+        etokens_h = torch.randint(0, 33, (8, 1024), generator=g)
         lens = torch.randint(128, 1025, (8,), generator=g)
-        emask = (torch.arange(1024)[None, :] >= lens[:, None]).to(dev)
+        emask_h = torch.arange(1024)[None, :] >= lens[:, None]
+        ecoords, etokens, emask = ecoords_h.to(dev), etokens_h.to(dev), emask_h.to(dev)
         with torch.no_grad():
             settle(torch, lambda: model(ecoords, etokens, emask))
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -332,7 +463,14 @@ def main():
             "workload": "WE + 33x512 embedding, 4 x (geometric MHA H=8 + LN + FFN 512-2048-512 GELU + LN), head to 20; "
                         "B=8 N=1024 lengths 128-1024, bf16 weights, fp32 WE (BASELINE.json configs[3])",
             "ms": e0.elapsed_time(e1) / 10, "valid_tokens": int(lens.sum()),
+            "tokens_per_s": float(lens.sum()) / (e0.elapsed_time(e1) / 10 * 1e-3),
         }
+        if not args.no_cpu:
+            with torch.no_grad():
+                dt, runs = cpu_timed(lambda: torch_oracle.encoder_forward_torch(state, min_spread, ecoords_h, etokens_h, emask_h), 20.0, 3)
+            result["encoder_forward"]["cpu_baseline"] = {
+                "value": float(lens.sum()) / dt, "unit": "valid tokens/s", "cores": threads, "kind": "port",
+                "sample": f"the full workload, median of {runs} run(s), the same weights in fp32 on the CPU PyTorch path, {dt:.1f} s"}
         # forward + backward of the same stack (cross-entropy on the unpadded tokens), no optimiser step
         model.train()
         labels = torch.randint(0, 20, (8, 1024), generator=g).to(dev)
@@ -352,17 +490,18 @@ def main():
         result["encoder_forward_backward"] = {"workload": "the same stack and batch, forward + backward (dropout 0)",
                                               "ms": e0.elapsed_time(e1) / 10}
 
-    # ---------------- CPU baseline: the tiled CPU PyTorch path on a bounded sample of observer rows ----------------
+    # ---------------- CPU baseline of the headline shape: the tiled CPU PyTorch path on a bounded sample of observer rows --------
     if not args.no_cpu:
-        from oracle import torch_oracle
-        threads = torch.get_num_threads()
-        rows = 64
-        t = time.perf_counter()
-        torch_oracle.we_torch(coords, wn, rows=list(range(rows)))
-        dt = time.perf_counter() - t
-        rows = int(max(64, min(N, rows * args.cpu_seconds / max(dt, 1e-3))))
-        rows -= rows % 64
-        sel = torch.linspace(0, N - 1, rows).long().tolist()
+        if args.full_cpu:
+            rows, sel = N, None
+        else:
+            rows = 64
+            t = time.perf_counter()
+            torch_oracle.we_torch(coords, wn, rows=list(range(rows)))
+            dt = time.perf_counter() - t
+            rows = int(max(64, min(N, rows * args.cpu_seconds / max(dt, 1e-3))))
+            rows -= rows % 64
+            sel = torch.linspace(0, N - 1, rows).long().tolist()
         t = time.perf_counter()
         torch_oracle.we_torch(coords, wn, rows=sel)
         dt = time.perf_counter() - t

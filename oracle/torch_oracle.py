@@ -236,3 +236,34 @@ def geo_attn_scalar_grad_mass(Q, K, V, dO, coords, sigma, key_padding_mask=None,
     if w_beta is None:
         return mass_sigma, None, total_sigma, None
     return mass_sigma, (spread * w_beta.abs()).sum(dim=(0, 2, 3)), total_sigma, (signed * w_beta).sum(dim=(0, 2, 3))
+
+
+def encoder_forward_torch(params, min_spread, coords, tokens, mask, attention=None):
+    """The encoder stack in fp32 on the CPU with the oracles in place of the kernels: WE(coords) + embedding[tokens],
+    then per layer geometric multi-head attention on the projections of x (per-head [d_model, d_k] weights and
+    [d_k] biases, sigma = min_spread + exp(w)), output projection, residual + LayerNorm, FFN (GELU), residual +
+    LayerNorm (old/old_scripts/encoder.py:33-41 and :88-89, old/old_scripts/attn/geometric_attn.py:625-655), and a
+    linear head.
+
+    params: state dict of the module (name -> tensor), any dtype; min_spread: float; attention: the attention oracle
+    to use, (Q, K, V, coords, sigma, mask) -> O [Z,H,N,d] (default: geo_attn_torch)."""
+    import torch.nn.functional as F
+    p = {k: v.detach().cpu().float() for k, v in params.items()}
+    if attention is None:
+        def attention(Q, K, V, c, sg, m):
+            return geo_attn_torch(Q, K, V, c, sg, m)[0]
+    wf, _, _ = we_torch(coords, torch.exp(p["wf_embedding.wavenumbers"]), mask)
+    x = wf + p["aa_embedding.weight"][tokens]
+    layers = 1 + max(int(k.split(".")[1]) for k in p if k.startswith("layers."))
+    for i in range(layers):
+        pre = f"layers.{i}."
+        Q, K, V = (torch.matmul(x.unsqueeze(1), p[pre + f"attn.{n}_proj"].unsqueeze(0)) + p[pre + f"attn.{n}_bias"][None, :, None]
+                   for n in ("q", "k", "v"))
+        O = attention(Q, K, V, coords, min_spread + torch.exp(p[pre + "attn.spread_weights"]), mask)
+        Z, H, N, d = O.shape
+        a = O.permute(0, 2, 3, 1).reshape(Z, N, H * d) @ p[pre + "attn.out_proj.weight"].T
+        x = F.layer_norm(x + a, (x.shape[-1],), p[pre + "attn_norm.weight"], p[pre + "attn_norm.bias"])
+        f = F.gelu(x @ p[pre + "ffn.in_proj.weight"].T + p[pre + "ffn.in_proj.bias"]) @ p[pre + "ffn.out_proj.weight"].T \
+            + p[pre + "ffn.out_proj.bias"]
+        x = F.layer_norm(x + f, (x.shape[-1],), p[pre + "ffn_norm.weight"], p[pre + "ffn_norm.bias"])
+    return x @ p["head.weight"].T + p["head.bias"]

@@ -12,27 +12,10 @@ pytestmark = pytest.mark.gpu
 
 
 def reference_forward(model, coords, tokens, mask):
-    """The same stack in fp32 on the CPU, with the oracles in place of the kernels."""
-    p = {k: v.detach().cpu().float() for k, v in model.state_dict().items()}
-    wn = torch.exp(p["wf_embedding.wavenumbers"])
-    wf, _, _ = torch_oracle.we_torch(coords, wn, mask)
-    x = wf + p["aa_embedding.weight"][tokens]
-    L = len(model.layers)
-    for i in range(L):
-        pre = f"layers.{i}."
-        xq = x
-        Q = torch.matmul(xq.unsqueeze(1), p[pre + "attn.q_proj"].unsqueeze(0)) + p[pre + "attn.q_bias"][None, :, None]
-        K = torch.matmul(xq.unsqueeze(1), p[pre + "attn.k_proj"].unsqueeze(0)) + p[pre + "attn.k_bias"][None, :, None]
-        V = torch.matmul(xq.unsqueeze(1), p[pre + "attn.v_proj"].unsqueeze(0)) + p[pre + "attn.v_bias"][None, :, None]
-        sig = model.layers[i].attn.min_spread + torch.exp(p[pre + "attn.spread_weights"])
-        O, _ = c_oracle.geo_attn(Q.numpy(), K.numpy(), V.numpy(), coords.numpy(), sig.numpy(), mask.numpy())
-        O = torch.from_numpy(O).float()
-        Z, H, N, d = O.shape
-        a = O.permute(0, 2, 3, 1).reshape(Z, N, H * d) @ p[pre + "attn.out_proj.weight"].T
-        x = F.layer_norm(x + a, (x.shape[-1],), p[pre + "attn_norm.weight"], p[pre + "attn_norm.bias"])
-        f = F.gelu(x @ p[pre + "ffn.in_proj.weight"].T + p[pre + "ffn.in_proj.bias"]) @ p[pre + "ffn.out_proj.weight"].T + p[pre + "ffn.out_proj.bias"]
-        x = F.layer_norm(x + f, (x.shape[-1],), p[pre + "ffn_norm.weight"], p[pre + "ffn_norm.bias"])
-    return x @ p["head.weight"].T + p["head.bias"]
+    """The same stack in fp32 on the CPU, with the oracles in place of the kernels (the C oracle for the attention)."""
+    def attention(Q, K, V, c, sg, m):
+        return torch.from_numpy(c_oracle.geo_attn(Q.numpy(), K.numpy(), V.numpy(), c.numpy(), sg.numpy(), m.numpy())[0]).float()
+    return torch_oracle.encoder_forward_torch(model.state_dict(), model.layers[0].attn.min_spread, coords, tokens, mask, attention)
 
 
 def test_small_encoder_matches_cpu_composition(gpu):
