@@ -417,7 +417,7 @@ def main():
             def bwd_step():
                 rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dOb.data_ptr(), acd.data_ptr(), sg.data_ptr(),
                                               None, None, L.data_ptr(), Dv.data_ptr(), dQ_.data_ptr(), dK_.data_ptr(), dV_.data_ptr(),
-                                              dsg.data_ptr(), None, 1, 8, 16384, 64, 0.0, 1.0, stream)
+                                              dsg.data_ptr(), None, 1, 8, 16384, 64, 0.0, 1.0, _lib.OPERAND_BF16, stream)
                 if rc != 0:
                     _lib.check(rc, "proteus_geo_attn_bwd")
             b_ms, _ = time_launches(torch, bwd_step, 5)

@@ -32,12 +32,17 @@ extern "C" {
 #define PROTEUS_OK                 0
 #define PROTEUS_ERR_NULL_POINTER  -1   /* a required pointer is NULL              */
 #define PROTEUS_ERR_BAD_SHAPE     -2   /* Z, N, K, H <= 0 or above the limits     */
-#define PROTEUS_ERR_BAD_HEAD_DIM  -3   /* d_head is not 64                        */
+#define PROTEUS_ERR_BAD_HEAD_DIM  -3   /* d_head is not 32, 64 or 128             */
 #define PROTEUS_ERR_BAD_LAYOUT    -4   /* unknown coords_layout value             */
 #define PROTEUS_ERR_BAD_ALIGNMENT -5   /* a pointer is not aligned as required    */
 #define PROTEUS_ERR_BAD_TUNING    -6   /* unknown tuning/variant selector         */
 #define PROTEUS_ERR_UNSUPPORTED   -7   /* legacy option not implemented           */
 #define PROTEUS_ERR_TOO_LARGE     -8   /* beyond the fixed capacity of an entry point that allocates nothing */
+#define PROTEUS_ERR_BAD_OPERAND_TYPE -9 /* operand_type is neither PROTEUS_OPERAND_BF16 nor PROTEUS_OPERAND_F16 */
+
+/* 16-bit type of Q, K, V (and dO) where an entry point takes an operand_type */
+#define PROTEUS_OPERAND_BF16 0
+#define PROTEUS_OPERAND_F16  1
 
 /* ---- coordinate layouts accepted by proteus_we_fwd ---- */
 #define PROTEUS_COORDS_SOA 0   /* [Z,3,N]: what the reference's wrapper hands its kernel */
@@ -215,11 +220,13 @@ int proteus_we_aniso_bwd_check(const float* d_out, const float* d_cb, const floa
  *   Padded query rows and rows without any valid key give O = 0, L = -inf
  *   (geometric_attn.py:196,233-236).
  *
- *   Q, K, V      [Z,H,N,64] bf16 (raw uint16 bit patterns), 16-byte aligned
+ *   Q, K, V      [Z,H,N,d_head] bf16 (raw uint16 bit patterns), 16-byte aligned; d_head = 32, 64 or 128
+ *                (the reference's kernel takes any d_k >= 16, geometric_attn.py:597; its test runs 32,
+ *                tests/attn/geo_attn.py:15-17), anything else returns PROTEUS_ERR_BAD_HEAD_DIM
  *   coords       [Z,N,3] f32
  *   sigma        [H] f32, > 0 (not checked on the device)
  *   key_pad_mask [Z,N] u8, non-zero = padded; may be NULL
- *   O            [Z,H,N,64] f32, 16-byte aligned
+ *   O            [Z,H,N,d_head] f32, 16-byte aligned
  *   L            [Z,H,N] f32; may be NULL (then not written)
  *   tuning       0 = automatic; otherwise a variant selector
  */
@@ -243,15 +250,17 @@ int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint1
  *     rbf   = exp(-|r_i - r_j|^2 / (2 sigma_h^2))
  *     s_ij  = S_ij + beta_h * (2 (rbf - min_rbf)/(max_rbf - min_rbf) - 1) * |S_ij|,   S_ij = q_i.k_j/sqrt(d)
  *     s_ij  = -inf where key j or query i is padded or rbf is outside [min_rbf, max_rbf]
- *   beta [H] f32; requires max_rbf > min_rbf.  Everything else as proteus_geo_attn_fwd
- *   (operands are bf16 here, fp16 in the reference).
+ *   beta [H] f32; requires max_rbf > min_rbf.
+ *   operand_type: PROTEUS_OPERAND_F16 reads Q, K, V as fp16 and runs the products on v_mfma_f32_32x32x16_f16, as
+ *   the reference does (it casts to fp16, geometric_attn.py:567-569); PROTEUS_OPERAND_BF16 as proteus_geo_attn_fwd.
+ *   Everything else as proteus_geo_attn_fwd.
  */
 int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                                 const float* coords, const float* sigma, const float* beta,
                                 const uint8_t* key_pad_mask,
                                 float* O, float* L,
                                 int Z, int H, int N, int d_head,
-                                float min_rbf, float max_rbf, int tuning, void* stream);
+                                float min_rbf, float max_rbf, int operand_type, int tuning, void* stream);
 
 /*
  * Backward of both attention forwards: dQ, dK, dV, d sigma (and d beta).
@@ -263,10 +272,11 @@ int proteus_geo_attn_legacy_fwd(const uint16_t* Q, const uint16_t* K, const uint
  * buffers.  beta == NULL selects the README logits (proteus_geo_attn_fwd), otherwise the
  * logits and pair mask of proteus_geo_attn_legacy_fwd.
  *
- *   Q, K, V, dO   [Z,H,N,64] bf16 (raw uint16), 16-byte aligned
+ *   Q, K, V, dO   [Z,H,N,d_head] (raw uint16), 16-byte aligned; d_head = 32, 64 or 128; bf16, or fp16 with
+ *                 operand_type = PROTEUS_OPERAND_F16 (legacy logits only: beta != NULL, else PROTEUS_ERR_BAD_OPERAND_TYPE)
  *   coords [Z,N,3] f32; sigma [H] f32; beta [H] f32 or NULL; key_pad_mask [Z,N] u8 or NULL
  *   L, D          [Z,H,N] f32
- *   dQ, dK, dV    [Z,H,N,64] f32, 16-byte aligned, fully overwritten (zeros at padded tokens)
+ *   dQ, dK, dV    [Z,H,N,d_head] f32, 16-byte aligned, fully overwritten (zeros at padded tokens)
  *   d_sigma       [H] f32, ACCUMULATED into with atomic adds (as the reference does, :541-543):
  *                 zero it first; may be NULL.  d_beta likewise (legacy logits only).
  */
@@ -274,7 +284,7 @@ int proteus_geo_attn_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          const float* coords, const float* sigma, const float* beta,
                          const uint8_t* key_pad_mask, const float* L, const float* D,
                          float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
-                         int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream);
+                         int Z, int H, int N, int d_head, float min_rbf, float max_rbf, int operand_type, void* stream);
 
 /* Validation half of proteus_geo_attn_bwd: same checks, no HIP call. */
 int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
@@ -282,10 +292,10 @@ int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint1
                                const uint8_t* key_pad_mask, const float* L, const float* D,
                                const float* dQ, const float* dK, const float* dV,
                                const float* d_sigma, const float* d_beta,
-                               int Z, int H, int N, int d_head, float min_rbf, float max_rbf);
+                               int Z, int H, int N, int d_head, float min_rbf, float max_rbf, int operand_type);
 
 /*
- * The same forward and backward on tensors that are not contiguous [Z,H,N,64].
+ * The same forward and backward on tensors that are not contiguous [Z,H,N,d_head].
  *
  * The reference's Triton launches take every tensor's strides
  * (old/old_scripts/attn/geometric_attn.py:588-599, :627-648); these entry
@@ -293,9 +303,9 @@ int proteus_geo_attn_bwd_check(const uint16_t* Q, const uint16_t* K, const uint1
  * being contiguous:
  *   forward   strides[12] : Q, K, V, O
  *   backward  strides[21] : Q, K, V, dO, dQ, dK, dV
- * so that slices of a fused [Z,N,3,H,64] projection are read in place and O or the
- * gradients are written in the memory order their consumer wants (e.g. [Z,N,H,64]).
- * Per tensor: token stride >= 64, no negative stride, batch / head stride 0 only for
+ * so that slices of a fused [Z,N,3,H,d] projection are read in place and O or the
+ * gradients are written in the memory order their consumer wants (e.g. [Z,N,H,d]).
+ * Per tensor: token stride >= d_head, no negative stride, batch / head stride 0 only for
  * Z == 1 / H == 1 (else PROTEUS_ERR_BAD_LAYOUT); every stride a multiple of 16 bytes
  * (PROTEUS_ERR_BAD_ALIGNMENT); N * token stride below 2^31 bytes (forward) or
  * 2^30 elements (backward) (PROTEUS_ERR_BAD_SHAPE).  coords, sigma, beta, the mask, L and D stay
@@ -317,20 +327,20 @@ int proteus_geo_attn_legacy_fwd_strided(const uint16_t* Q, const uint16_t* K, co
                                         const uint8_t* key_pad_mask,
                                         float* O, float* L,
                                         int Z, int H, int N, int d_head,
-                                        float min_rbf, float max_rbf, int tuning, void* stream);
+                                        float min_rbf, float max_rbf, int operand_type, int tuning, void* stream);
 int proteus_geo_attn_bwd_strided(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
                                  const int64_t* strides,
                                  const float* coords, const float* sigma, const float* beta,
                                  const uint8_t* key_pad_mask, const float* L, const float* D,
                                  float* dQ, float* dK, float* dV, float* d_sigma, float* d_beta,
-                                 int Z, int H, int N, int d_head, float min_rbf, float max_rbf, void* stream);
+                                 int Z, int H, int N, int d_head, float min_rbf, float max_rbf, int operand_type, void* stream);
 int proteus_geo_attn_bwd_strided_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* dO,
                                        const int64_t* strides,
                                        const float* coords, const float* sigma, const float* beta,
                                        const uint8_t* key_pad_mask, const float* L, const float* D,
                                        const float* dQ, const float* dK, const float* dV,
                                        const float* d_sigma, const float* d_beta,
-                                       int Z, int H, int N, int d_head, float min_rbf, float max_rbf);
+                                       int Z, int H, int N, int d_head, float min_rbf, float max_rbf, int operand_type);
 
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);

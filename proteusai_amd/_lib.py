@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "libproteus_hip.so")
 
 COORDS_SOA = 0
 COORDS_AOS = 1
+OPERAND_BF16, OPERAND_F16 = 0, 1     # PROTEUS_OPERAND_* of include/proteus_hip.h
 
 # every symbol include/proteus_hip.h declares
 SYMBOLS = [
@@ -80,12 +81,12 @@ def load():
     lib.proteus_geo_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     lib.proteus_geo_attn_legacy_fwd.restype = ci
     lib.proteus_geo_attn_legacy_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci,
-                                                ctypes.c_float, ctypes.c_float, ci, vp]
+                                                ctypes.c_float, ctypes.c_float, ci, ci, vp]
     cf = ctypes.c_float
     lib.proteus_geo_attn_bwd.restype = ci
-    lib.proteus_geo_attn_bwd.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf, vp]
+    lib.proteus_geo_attn_bwd.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf, ci, vp]
     lib.proteus_geo_attn_bwd_check.restype = ci
-    lib.proteus_geo_attn_bwd_check.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf]
+    lib.proteus_geo_attn_bwd_check.argtypes = [vp] * 15 + [ci, ci, ci, ci, cf, cf, ci]
     i64p = ctypes.POINTER(ctypes.c_int64)
     lib.proteus_geo_attn_fwd_strided.restype = ci
     lib.proteus_geo_attn_fwd_strided.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
@@ -93,11 +94,11 @@ def load():
     lib.proteus_geo_attn_fwd_strided_check.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_legacy_fwd_strided.restype = ci
     lib.proteus_geo_attn_legacy_fwd_strided.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci,
-                                                        ctypes.c_float, ctypes.c_float, ci, vp]
+                                                        ctypes.c_float, ctypes.c_float, ci, ci, vp]
     lib.proteus_geo_attn_bwd_strided.restype = ci
-    lib.proteus_geo_attn_bwd_strided.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, vp]
+    lib.proteus_geo_attn_bwd_strided.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, ci, vp]
     lib.proteus_geo_attn_bwd_strided_check.restype = ci
-    lib.proteus_geo_attn_bwd_strided_check.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf]
+    lib.proteus_geo_attn_bwd_strided_check.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, ci]
     lib.proteus_geo_attn_fwd_check.restype = ci
     lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_num_variants.restype = ci

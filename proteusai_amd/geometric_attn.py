@@ -24,13 +24,23 @@ def _rows_ok(t, itemsize):
             and t.size(2) * t.stride(2) * itemsize < 2 ** 31)
 
 
-def _operand(t):
-    """bf16 view of an operand the kernels can read where it lies (a copy only if it has to be cast or its rows
+def _operand(t, dtype=torch.bfloat16):
+    """16-bit view of an operand the kernels can read where it lies (a copy only if it has to be cast or its rows
     are not contiguous)."""
     t = t.detach()
-    if t.dtype != torch.bfloat16:
-        t = t.to(torch.bfloat16)
+    if t.dtype != dtype:
+        t = t.to(dtype)
     return t if _rows_ok(t, 2) else t.contiguous()
+
+
+def _operand_type(operand_dtype, legacy):
+    if operand_dtype in (None, torch.bfloat16):
+        return torch.bfloat16, _lib.OPERAND_BF16
+    if operand_dtype == torch.float16:
+        if not legacy:
+            raise NotImplementedError("fp16 operands go with the beta-weighted logits (pass betas); the README logits run in bf16")
+        return torch.float16, _lib.OPERAND_F16
+    raise AssertionError(f"operand_dtype must be torch.bfloat16 or torch.float16, not {operand_dtype}")
 
 
 def _is_plain(*ts):
@@ -39,11 +49,12 @@ def _is_plain(*ts):
 
 def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = False, tuning: int = 0,
              betas=None, min_rbf: float = 0.0, max_rbf: float = 1.0, check_sigma: bool = True,
-             token_major_out: bool = False):
-    """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None).
+             token_major_out: bool = False, operand_dtype=None):
+    """O = geo_attn(Q, K, V [Z,H,N,d], coords [Z,N,3], sigma [H], key_padding_mask [Z,N] bool | None), d = 32, 64 or 128.
 
-    Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569),
-    coords and sigma to fp32; O is fp32 [Z,H,N,d] as in the reference (:578).
+    Operands are cast to bf16 (the reference casts to fp16, geometric_attn.py:567-569; with `betas`,
+    operand_dtype=torch.float16 does the same here), coords and sigma to fp32; O is fp32 [Z,H,N,d] as in the
+    reference (:578).
     key_padding_mask: True = padded.  Padded query rows and rows without a
     valid key give O = 0 and logsumexp = -inf.  With return_lse the
     logsumexp L [Z,H,N] is returned as well.
@@ -74,7 +85,8 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     lib = _lib.load()
     dev = Q.device
     legacy = betas is not None
-    q, k, v = _operand(Q), _operand(K), _operand(V)
+    op_dtype, op_type = _operand_type(operand_dtype, legacy)
+    q, k, v = _operand(Q, op_dtype), _operand(K, op_dtype), _operand(V, op_dtype)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
     m = None
@@ -107,32 +119,34 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
                 rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
                                                      bt.data_ptr(), None if m is None else m.data_ptr(),
                                                      O.data_ptr(), L.data_ptr(), Z, H, N, d,
-                                                     float(min_rbf), float(max_rbf), int(tuning), stream)
+                                                     float(min_rbf), float(max_rbf), op_type, int(tuning), stream)
             else:
                 rc = lib.proteus_geo_attn_legacy_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                                              _lib.stride_array(q, k, v, O), c.data_ptr(), s.data_ptr(),
                                                              bt.data_ptr(), None if m is None else m.data_ptr(),
                                                              O.data_ptr(), L.data_ptr(), Z, H, N, d,
-                                                             float(min_rbf), float(max_rbf), int(tuning), stream)
+                                                             float(min_rbf), float(max_rbf), op_type, int(tuning), stream)
     _lib.check(rc, "proteus_geo_attn_fwd")
     return (O, L) if return_lse else O
 
 
 def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, betas=None,
-                      min_rbf: float = 0.0, max_rbf: float = 1.0):
+                      min_rbf: float = 0.0, max_rbf: float = 1.0, operand_dtype=None):
     """dQ, dK, dV [Z,H,N,d] f32, d_sigma [H] f32, d_betas [H] f32 | None from the forward's O and logsumexp L.
 
     What the reference's wrapper does around its backward kernel (geometric_attn.py:609-660):
-    D = rowsum(O*dO), dO cast to the operand type (bf16 here), zeroed accumulators for the per-head scalars.
+    D = rowsum(O*dO), dO cast to the operand type (bf16, or fp16 with operand_dtype=torch.float16 and betas), zeroed
+    accumulators for the per-head scalars.
     """
     Z, H, N, d = Q.shape
     if not Q.is_cuda:
         raise _lib.ProteusError("geo_attn_backward needs tensors on the GPU (there is no CPU path)")
     lib = _lib.load()
     dev = Q.device
-    q, k, v = _operand(Q), _operand(K), _operand(V)
+    op_dtype, op_type = _operand_type(operand_dtype, betas is not None)
+    q, k, v = _operand(Q, op_dtype), _operand(K, op_dtype), _operand(V, op_dtype)
     D = torch.sum(O.detach().float() * dO.detach(), dim=3).contiguous()       # fp32 by type promotion
-    do = _operand(dO)
+    do = _operand(dO, op_dtype)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
     lse = L.detach().to(torch.float32).contiguous()
@@ -154,7 +168,7 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
         tail = (c.data_ptr(), s.data_ptr(), None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
                 lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
                 d_sigma.data_ptr(), None if d_beta is None else d_beta.data_ptr(),
-                Z, H, N, d, float(min_rbf), float(max_rbf), stream)
+                Z, H, N, d, float(min_rbf), float(max_rbf), op_type, stream)
         if _is_plain(q, k, v, do, dQ, dK, dV):
             rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), *tail)
         else:
@@ -170,11 +184,12 @@ class _geometric_attn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, Q, K, V, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf, check_sigma=True,
-                token_major_out=False, out_dtype=None):
+                token_major_out=False, out_dtype=None, operand_dtype=None):
         O, L = geo_attn(Q, K, V, coords, spreads, key_padding_mask, return_lse=True, betas=betas,
-                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma, token_major_out=token_major_out)
+                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma, token_major_out=token_major_out,
+                        operand_dtype=operand_dtype)
         ctx.save_for_backward(Q, K, V, O, L, coords, spreads, betas, key_padding_mask)
-        ctx.min_rbf, ctx.max_rbf = min_rbf, max_rbf
+        ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype = min_rbf, max_rbf, operand_dtype
         # the fp32 O is what the backward reads; the caller may ask for it in its own working precision
         return O if out_dtype is None or out_dtype == O.dtype else O.to(out_dtype)
 
@@ -182,13 +197,13 @@ class _geometric_attn(torch.autograd.Function):
     def backward(ctx, dO):
         Q, K, V, O, L, coords, spreads, betas, mask = ctx.saved_tensors
         dQ, dK, dV, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
-                                                        ctx.min_rbf, ctx.max_rbf)
+                                                        ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype)
         return (dQ.to(Q.dtype), dK.to(K.dtype), dV.to(V.dtype), None, d_sigma.to(spreads.dtype),
-                None if betas is None else d_beta.to(betas.dtype), None, None, None, None, None, None)
+                None if betas is None else d_beta.to(betas.dtype), None, None, None, None, None, None, None)
 
 
 def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True,
-                   token_major_out=False, out_dtype=None):
+                   token_major_out=False, out_dtype=None, operand_dtype=None):
     """Same call as the reference's geometric_attn (geometric_attn.py:545-548).
 
     betas=None selects the README logits S*(1+RBF) (README.md:40; the rbf range must then be the full
@@ -196,12 +211,13 @@ def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00
     [min_rbf, max_rbf] pair mask (geometric_attn.py:193-201).
 
     Beyond the reference's call: token_major_out lays O out [Z,N,H,d] in memory (returned as a [Z,H,N,d] view),
-    out_dtype returns O in another dtype than fp32 (the fp32 result is kept for the backward either way).
+    out_dtype returns O in another dtype than fp32 (the fp32 result is kept for the backward either way),
+    operand_dtype=torch.float16 (with betas) casts Q, K, V and dO to fp16 as the reference does (:567-569) instead of bf16.
     """
     if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
         raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
     return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads,
-                                 token_major_out, out_dtype)
+                                 token_major_out, out_dtype, operand_dtype)
 
 
 class GeoAttention(nn.Module):

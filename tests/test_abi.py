@@ -29,7 +29,7 @@ def test_version_and_strerror():
     lib = _lib.load()
     assert lib.proteus_version() >= 100
     assert lib.proteus_strerror(0) == b"ok"
-    for code in range(-8, 0):
+    for code in range(-9, 0):
         assert lib.proteus_strerror(code) not in (b"", b"unknown error code")
     assert lib.proteus_strerror(-99) == b"unknown error code"
 
@@ -96,20 +96,24 @@ def test_attention_argument_validation():
     assert call(7, None) == 0                  # L is optional
     for idx in (8, 9, 10):
         assert call(idx, 0) == -2
-    assert call(11, 32) == -3 and call(11, 128) == -3
+    assert call(11, 32) == 0 and call(11, 128) == 0          # head dimensions 32, 64, 128
+    assert call(11, 48) == -3 and call(11, 16) == -3 and call(11, 256) == -3
     assert call(12, 55) == -6
     assert call(0, p + 2) == -5
     assert lib.proteus_geo_attn_fwd(p, p, p, p, p, None, p, p, 1, 2, 16, 48, 0, None) == -3
     # legacy-logits entry point: same checks, plus beta and the rbf range
-    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, None, None, p, p, 1, 2, 16, 64, 0.0, 1.0, 0, None) == -1
-    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0.5, 0.5, 0, None) == -2
-    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 32, 0.0, 1.0, 0, None) == -3
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, None, None, p, p, 1, 2, 16, 64, 0.0, 1.0, 0, 0, None) == -1
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0.5, 0.5, 0, 0, None) == -2
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 48, 0.0, 1.0, 0, 0, None) == -3
+    # ... and the operand type: bf16 (0) or fp16 (1)
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0.0, 1.0, 2, 0, None) == -9
+    assert lib.proteus_geo_attn_legacy_fwd(p, p, p, p, p, p, None, p, p, 1, 2, 16, 64, 0.0, 1.0, -1, 0, None) == -9
 
 
 def test_attention_backward_argument_validation():
     lib = _lib.load()
     p = 0x1000
-    ok = [p, p, p, p, p, p, None, None, p, p, p, p, p, p, None, 1, 2, 16, 64, 0.0, 1.0]
+    ok = [p, p, p, p, p, p, None, None, p, p, p, p, p, p, None, 1, 2, 16, 64, 0.0, 1.0, 0]
 
     def call(**kw):
         a = list(ok)
@@ -120,7 +124,9 @@ def test_attention_backward_argument_validation():
     for i in (0, 1, 2, 3, 4, 5, 8, 9, 10, 11, 12):
         assert call(**{f"a{i}": None}) == -1
     assert call(a15=0) == -2 and call(a17=(1 << 20) + 1) == -2
-    assert call(a18=32) == -3
+    assert call(a18=32) == 0 and call(a18=128) == 0 and call(a18=48) == -3
+    assert call(a21=1) == -9 and call(a21=2) == -9      # fp16 operands go with the legacy logits (beta) only
+    assert call(a6=p, a21=1) == 0 and call(a6=p, a21=2) == -9
     assert call(a10=p + 4) == -5
     assert call(a6=p, a19=0.5, a20=0.5) == -2          # legacy logits need max_rbf > min_rbf
     assert lib.proteus_geo_attn_bwd(*(ok[:3] + [None] + ok[4:] + [None])) == -1
@@ -290,7 +296,7 @@ def test_strided_attention_argument_validation():
 
     def bwd(st):
         return lib.proteus_geo_attn_bwd_strided_check(p, p, p, p, st, p, p, None, None, p, p, p, p, p, p, None,
-                                                      Z, H, N, 64, 0.0, 1.0)
+                                                      Z, H, N, 64, 0.0, 1.0, 0)
     assert bwd(arr(*(plain * 7))) == 0
     assert bwd(arr(*(fused * 3 + tok * 4))) == 0
     assert bwd(None) == -1

@@ -56,17 +56,20 @@ def test_attention_forward_and_backward(gpu, case):
     Z, H, N = int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.integers(1, 400))
     g = torch.Generator().manual_seed(3000 + case)
     qs = float(rng.choice([0.5, 1.0, 2.0]))
-    Q = (torch.randn(Z, H, N, 64, generator=g) * qs).bfloat16()
-    K = torch.randn(Z, H, N, 64, generator=g).bfloat16()
-    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
-    dO = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    d = (64, 32, 64, 128)[case % 4]                       # head dimension
+    legacy = case % 3 == 2
+    op = torch.float16 if legacy and case % 5 == 0 else torch.bfloat16      # operand type (fp16 goes with the legacy logits)
+    Q = (torch.randn(Z, H, N, d, generator=g) * qs).to(op)
+    K = torch.randn(Z, H, N, d, generator=g).to(op)
+    V = torch.randn(Z, H, N, d, generator=g).to(op)
+    dO = torch.randn(Z, H, N, d, generator=g).to(op)
     coords = chain(rng, Z, N, float(rng.choice([0.5, 1.0, 3.0])), rng.normal(size=3) * float(rng.choice([0.0, 100.0, 3000.0])))
     sigma = torch.from_numpy(rng.uniform(1.0, 30.0, H).astype(np.float32))
     mask = torch.from_numpy(rng.random((Z, N)) < float(rng.choice([0.0, 0.2, 0.7])))
-    legacy = case % 3 == 2
     betas = torch.from_numpy(rng.uniform(0.1, 2.0, H).astype(np.float32)) if legacy else None
     lo, hi = (0.02, 0.95) if legacy and case % 2 == 0 else (0.0, 1.0)
-    what = f"case {case}: Z={Z} H={H} N={N} legacy={legacy}"
+    what = f"case {case}: Z={Z} H={H} N={N} d={d} legacy={legacy} {op}"
+    op_arg = op if legacy else None
 
     s = sigma.to(gpu).requires_grad_(True)
     bt = None if betas is None else betas.to(gpu).requires_grad_(True)
@@ -76,13 +79,13 @@ def test_attention_forward_and_backward(gpu, case):
         # operands as slices of one fused [Z,N,3,H,d] buffer, O token-major: read and written in place
         fused = torch.stack([t.permute(0, 2, 1, 3) for t in (Q, K, V)], dim=2).contiguous().to(gpu).requires_grad_(True)
         q, k, v = (fused[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi, token_major_out=True)
+        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi, token_major_out=True, operand_dtype=op_arg)
         assert O.permute(0, 2, 1, 3).is_contiguous()
         O.backward(dO.to(gpu).float())
         gq, gk, gv = (fused.grad[:, :, i].permute(0, 2, 1, 3) for i in range(3))
     else:
         q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
-        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi)
+        O = pa.geometric_attn(q, k, v, coords.to(gpu), s, bt, mask.to(gpu), lo, hi, operand_dtype=op_arg)
         O.backward(dO.to(gpu).float())
         gq, gk, gv = q.grad, k.grad, v.grad
 
@@ -118,7 +121,7 @@ def test_attention_forward_and_backward(gpu, case):
             f"{what} {name}: error / pair mass {(err / pair_mass.clamp_min(1e-300)).max():.3e}"
         if (total.abs() >= 0.25 * pair_mass).all() and total.norm() > 1e-9:
             assert rel_l2(gg.numpy(), total.numpy()) <= 1e-2, f"{what} {name}: {rel_l2(gg.numpy(), total.numpy()):.3e}"
-    if not legacy:
+    if not legacy and d == 64:
         # the software-pipelined forward is the default only for large grids: force it on the same inputs
         O5 = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), tuning=5).cpu().double()
         assert torch.isfinite(O5).all(), what
