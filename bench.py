@@ -115,6 +115,20 @@ def probe_rates(lib, torch, dev):
     return rates
 
 
+def probe_slot_ms(lib, torch, dev, mode, blocks=512, iters=4000):
+    """Seconds per slot per SIMD of the co-issue probe (a slot = one 32x32x16 bf16 product + the softmax work of two
+    scores) at two waves per SIMD: blocks x 4 waves x iters x 8 slots over 1024 SIMDs."""
+    sink = torch.empty(blocks * 256, device=dev)
+    lib.proteus_probe_mfma_softmax_slot(mode, blocks, iters, sink.data_ptr(), None)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    lib.proteus_probe_mfma_softmax_slot(mode, blocks, iters, sink.data_ptr(), None)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / (blocks * 4 * iters * 8 / 1024.0)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -390,6 +404,17 @@ def main():
             "roofline": {"kernel": "geo_attn_fwd_pipe_kernel", "bound": "mfma", "achieved": a_tflops, "peak": PEAK_BF16_MFMA_TFLOPS,
                          "unit": "TFLOP/s", "frac": a_tflops / PEAK_BF16_MFMA_TFLOPS,
                          "traffic": a_traffic, "traffic_source": a_traffic_src},
+        }
+        # Issue model: the kernel's inner loop is eight "slots" per 32 x 32 block of pairs (8 matrix products: 4 for the
+        # scores, 4 for P V), each with the softmax work of two scores per lane.  The probe measures what one SIMD needs per
+        # slot at the kernel's occupancy (two waves) when it does nothing else: no staging, no geometry, no barrier.
+        slots = 8.0 * 8 * (16384 / 32) * (16384 / 32) / 1024.0               # per SIMD
+        t_m, t_v, t_b = (probe_slot_ms(lib, torch, dev, m) for m in (0, 1, 2))
+        leg["roofline"]["issue_model"] = {
+            "slot": "one 32x32x16 bf16 product + 2 fma + 2 exp2 + 1 pack + 1 packed add, two waves per SIMD",
+            "ns_per_slot_per_simd": {"matrix_only": t_m * 1e9, "vector_only": t_v * 1e9, "both": t_b * 1e9},
+            "model_ms": slots * t_b * 1e3, "frac": slots * t_b * 1e3 / a_ms,
+            "matrix_only_ms": slots * t_m * 1e3,
         }
         pa_ = read_profile(PROFILE_ATTN)
         if "mfma_util" in pa_:

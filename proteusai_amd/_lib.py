@@ -24,7 +24,7 @@ SYMBOLS = [
     "proteus_geo_attn_legacy_fwd_strided",
     "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
-    "proteus_probe_valu_rate", "proteus_probe_sincos",
+    "proteus_probe_valu_rate", "proteus_probe_sincos", "proteus_probe_mfma_softmax_slot",
 ]
 
 _lib = None
@@ -108,6 +108,8 @@ def load():
     lib.proteus_probe_valu_rate.argtypes = [ci, ci, ci, vp, vp]
     lib.proteus_probe_sincos.restype = ci
     lib.proteus_probe_sincos.argtypes = [vp, vp, vp, vp, ci, ci, vp]
+    lib.proteus_probe_mfma_softmax_slot.restype = ci
+    lib.proteus_probe_mfma_softmax_slot.argtypes = [ci, ci, ci, vp, vp]
     _lib = lib
     return lib
 

@@ -1,5 +1,6 @@
 // Instruction-rate and accuracy probes (not on the product path): they state, from measurement, the denominators
-// the WE roofline model uses and the error of the hardware sin/cos/rsq path.
+// the WE roofline model uses, the error of the hardware sin/cos/rsq path, and how far one matrix product and the
+// softmax work that goes with it overlap on a SIMD (the issue model of the attention kernel).
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -80,7 +81,60 @@ __global__ void sincos_probe_kernel(const float* x, float* s, float* c, float* q
     q[i] = __builtin_fmaf(e, 0.5f * inv, r0);
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float  floatx16 __attribute__((ext_vector_type(16)));
+typedef float  floatx2 __attribute__((ext_vector_type(2)));
+
+// One "slot" of the attention forward's inner loop: a 32x32x16 bf16 matrix product and the softmax work of two scores
+// (two fused multiply-adds, two exp2, one pack to bf16, one packed row-sum add).  MODE 0: the products only;
+// 1: the vector work only; 2: both, in the order the kernel issues them.  Eight slots per loop trip.
+template <int MODE>
+__global__ __launch_bounds__(256)
+void mfma_softmax_slot_kernel(float* sink, int iters) {
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    bf16x8 a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { a[e] = (__bf16)(0.001f * (float)(threadIdx.x + e)); b[e] = (__bf16)(0.002f * (float)(e + 1)); }
+    float s0 = 0.001f * (float)threadIdx.x, s1 = 0.5f - s0, lsum = 0.f;
+    float log2e = 1.4426950408889634f, mneg = -0.25f;
+    asm volatile("" : "+v"(log2e), "+v"(mneg));
+#pragma unroll 1
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (MODE != 1) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+            if (MODE != 0) {
+                asm volatile("" : "+v"(s0), "+v"(s1));          // opaque: nothing of the step is hoisted out of the loop
+                const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0, log2e, mneg));
+                const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1, log2e, mneg));
+                const floatx2 f = {x0, x1};
+                const bf16x2 pk = __builtin_convertvector(f, bf16x2);
+                lsum = __builtin_amdgcn_fdot2_f32_bf16(pk, __builtin_bit_cast(bf16x2, 0x3f803f80u), lsum, false);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float s = lsum;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[r];
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 }  // namespace
+
+extern "C" int proteus_probe_mfma_softmax_slot(int mode, int blocks, int iters, float* sink, void* stream) {
+    if (!sink) return PROTEUS_ERR_NULL_POINTER;
+    if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return PROTEUS_ERR_BAD_SHAPE;
+    if (mode < 0 || mode > 2) return PROTEUS_ERR_BAD_TUNING;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (mode == 0)      hipLaunchKernelGGL((mfma_softmax_slot_kernel<0>), dim3(blocks), dim3(256), 0, st, sink, iters);
+    else if (mode == 1) hipLaunchKernelGGL((mfma_softmax_slot_kernel<1>), dim3(blocks), dim3(256), 0, st, sink, iters);
+    else                hipLaunchKernelGGL((mfma_softmax_slot_kernel<2>), dim3(blocks), dim3(256), 0, st, sink, iters);
+    return (int)hipGetLastError();
+}
 
 extern "C" int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;

@@ -59,6 +59,52 @@ def test_cfg4_shape_bf16_and_padding_independence(gpu):
     assert torch.equal(out[valid], out2[valid])
 
 
+def test_cfg4_shape_embedding_and_first_attention_on_sampled_rows(gpu):
+    """At the real shape (B=8, N=1024, d_model=512, H=8, bf16 weights, fp32 WE, lengths in [128, 1024]) a dense oracle of
+    the whole stack takes too long for a test, but rows are independent in both kernels: the embedding and the first
+    layer's attention (fed with the activations the model itself produces) are checked on sampled rows."""
+    torch.manual_seed(4)
+    model = pa.ProteusEncoder().eval().to(gpu)
+    model.aa_embedding.to(torch.bfloat16)
+    model.layers.to(torch.bfloat16)
+    model.head.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(4)
+    coords = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)])
+    tokens = torch.randint(0, 33, (8, 1024), generator=g)
+    lens = torch.randint(128, 1025, (8,), generator=g)
+    mask = torch.arange(1024)[None, :] >= lens[:, None]
+    rows = sorted(set(torch.randint(0, 1024, (40,), generator=g).tolist()) | {0, 127, 128, 1023})
+    with torch.no_grad():
+        wf = model.wf_embedding(coords.to(gpu), None, key_padding_mask=mask.to(gpu))
+        wn = torch.exp(model.wf_embedding.wavenumbers.detach()).cpu()
+        ref_wf, _, _ = c_oracle.we(coords.numpy(), wn.numpy(), mask.numpy(), rows=rows)
+        got_wf = wf.cpu().numpy()[:, rows]
+        assert np.isfinite(got_wf).all()
+        e = np.linalg.norm(got_wf - ref_wf) / np.linalg.norm(ref_wf)
+        assert e <= 1e-4, f"embedding at the encoder's shape: rel-L2 {e:.3e}"
+        assert (got_wf[mask.numpy()[:, rows]] == 0).all()
+
+        attn = model.layers[0].attn
+        x = (wf + model.aa_embedding(tokens.to(gpu)).to(wf.dtype)).to(torch.bfloat16)
+        w, b = attn._fused_qkv()
+        qkv = torch.addmm(b, x.reshape(8 * 1024, 512), w).view(8, 1024, 3, 8, 64)
+        Q, K, V = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))              # strided [Z,H,N,d] views, read in place
+        sigma = attn.get_spreads().detach().float()
+        O, L = pa.geo_attn(Q, K, V, coords.to(gpu), sigma, mask.to(gpu), return_lse=True)
+        Or, Lr = c_oracle.geo_attn(Q.float().cpu().numpy(), K.float().cpu().numpy(), V.float().cpu().numpy(), coords.numpy(),
+                                   sigma.cpu().numpy(), mask.numpy(), rows=rows)
+        O, L = O.cpu().numpy()[:, :, rows].astype(np.float64), L.cpu().numpy()[:, :, rows].astype(np.float64)
+        fin = np.isfinite(Lr)
+        assert np.isfinite(O).all() and (np.isneginf(L) == ~fin).all()
+        # O is a convex combination of V rows whose weights are rounded to bf16: the 2e-2 bar of unit-scale values scales
+        # with the largest |V| (the projections of WE + embedding reach about 10 here)
+        vmax = float(V.float().abs().max())
+        assert 1.0 < vmax < 100.0
+        assert np.abs(O - Or).max() <= 2e-2 * vmax / 4, f"first-layer attention at the encoder's shape: {np.abs(O - Or).max():.3e} (max |V| {vmax:.2f})"
+        assert np.abs(L[fin] - Lr[fin]).max() <= 4e-3
+        assert (O[~fin] == 0).all()
+
+
 def test_training_step_through_both_kernels(gpu):
     # forward and backward of the whole stack on the HIP kernels (attention backward, wavenumber backward of the
     # embedding), one SGD step, and the loss goes down
