@@ -132,9 +132,9 @@ template <int KT, bool SPLIT, bool FRACT, int MAG>
 __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_red,
                                         const float* __restrict__ cz, const uint8_t* __restrict__ mz, const int layout,
                                         float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
-                                        const int N, const int K, const size_t zN,
+                                        const int N, const int j_end, const int K, const size_t zN,
                                         const int tid, const int lane, const int wave,
-                                        const int i, const bool i_in, const bool i_valid, const bool any_valid,
+                                        const int i, const bool i_in, const bool i_valid,
                                         const float xi, const float yi, const float zi,
                                         const int k0, const bool wave_active, const float (&kr)[KT])
 {
@@ -143,8 +143,7 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
     for (int t = 0; t < KT; ++t) { acc_oc[t] = 0.f; acc_os[t] = 0.f; acc_c[t] = 0.f; acc_s[t] = 0.f; }
     float nzero = 0.f;
 
-    if (any_valid) {
-        const int j_end = N;
+    {
         for (int jb = 0; jb < j_end; jb += WE_JB) {
             // -- stage one block of sources, keeping only the unpadded ones --
             const int  j    = jb + tid;
@@ -244,6 +243,23 @@ __device__ __forceinline__ void we_body(float4* s_keys, int* s_wcount, float* s_
     }
 }
 
+// Rows of 64 observers that are all padded: zeros for the wavenumbers this wave (this workgroup, with SPLIT: its
+// wave 0) is responsible for.
+template <int KT, bool SPLIT, int MAG>
+__device__ __forceinline__ void we_write_zero_rows(float* __restrict__ out, float* __restrict__ cos_sums, float* __restrict__ sin_sums,
+                                                   const int K, const size_t zN, const int i, const bool i_in, const int wave, const int ytile)
+{
+    if (SPLIT && wave > 0) return;
+    const int k0 = SPLIT ? ytile * KT : (ytile * WE_WAVES + wave) * KT;
+    if (k0 >= K || !i_in) return;
+    const size_t row = zN + (size_t)i;
+    float* o = out + row * (size_t)(2 * K) + 2 * (size_t)k0;
+    for (int t = 0; t < KT && k0 + t < K; ++t) {
+        o[2 * t] = 0.0f; o[2 * t + 1] = 0.0f;
+        if (MAG != WE_MAG_NO_SUMS) { cos_sums[row * (size_t)K + k0 + t] = 0.0f; sin_sums[row * (size_t)K + k0 + t] = 0.0f; }
+    }
+}
+
 // KT     wavenumbers per wave (4*KT accumulators per lane)
 // SPLIT  small problems: the four waves of a workgroup share ONE wavenumber tile and split the staged
 //        sources between them (wave w takes sources w, w+4, ...); the partial sums meet in LDS at the
@@ -261,6 +277,7 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     __shared__ float4 s_keys[WE_JB + WE_WAVES];   // padding: the stream loop reads one step ahead
     __shared__ int    s_wcount[WE_WAVES];
     __shared__ float  s_box[WE_WAVES][6];
+    __shared__ int    s_last[WE_WAVES];
     __shared__ float  s_red[SPLIT ? (4 * KT + 1) * 64 : 1];
 
     const int tid  = threadIdx.x;
@@ -286,6 +303,12 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     // Every wave of the workgroup sees the same 64 observers, so this exit is
     // uniform over the workgroup and happens before the first barrier.
     const bool any_valid = __builtin_amdgcn_ballot_w64(i_valid) != 0;
+    if (!any_valid) {
+        // 64 padded (or out-of-range) observers: zeros, and nothing else to do (in a batch of ragged lengths this is a
+        // large share of the workgroups)
+        we_write_zero_rows<KT, SPLIT, MAG>(out, cos_sums, sin_sums, K, zN, i, i_in, wave, blockIdx.y);
+        return;
+    }
 
     // ---- this wave's wavenumbers, converted to revolutions per angstrom ----
     const int  k0          = SPLIT ? blockIdx.y * KT : (blockIdx.y * WE_WAVES + wave) * KT;
@@ -303,11 +326,16 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
 
     // ---- can any phase of this wave leave the +-256 revolutions v_sin/v_cos accept? ----
     bool wg_safe = false;
-    // Bounding box of all coordinates of the batch item (a few loads per thread, once), then the
-    // distance from each observer to its farthest corner bounds every r_ij of the lane.
+    // Bounding box of the unpadded coordinates of the batch item (a few loads per thread, once), then the
+    // distance from each observer to its farthest corner bounds every r_ij of the lane.  The same pass finds
+    // where the unpadded sources end: the blocks of sources behind that are never staged.
+    int j_end = 0;
     {
         float lo[3] = {3.0e38f, 3.0e38f, 3.0e38f}, hi[3] = {-3.0e38f, -3.0e38f, -3.0e38f};
+        int last = 0;
         for (int j = tid; j < N; j += WE_THREADS) {
+            if (mz && mz[j]) continue;
+            last = j + 1;
             float p[3];
             if (layout == PROTEUS_COORDS_SOA) { p[0] = cz[j]; p[1] = cz[(size_t)N + j]; p[2] = cz[2 * (size_t)N + j]; }
             else                              { p[0] = cz[3 * (size_t)j]; p[1] = cz[3 * (size_t)j + 1]; p[2] = cz[3 * (size_t)j + 2]; }
@@ -317,11 +345,14 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
 #pragma unroll
         for (int c = 0; c < 3; ++c)
             for (int o = 32; o > 0; o >>= 1) { lo[c] = fminf(lo[c], __shfl_xor(lo[c], o)); hi[c] = fmaxf(hi[c], __shfl_xor(hi[c], o)); }
+        for (int o = 32; o > 0; o >>= 1) last = max(last, __shfl_xor(last, o));
         if (lane == 0) {
 #pragma unroll
             for (int c = 0; c < 3; ++c) { s_box[wave][c] = lo[c]; s_box[wave][3 + c] = hi[c]; }
+            s_last[wave] = last;
         }
         __syncthreads();
+        j_end = max(max(s_last[0], s_last[1]), max(s_last[2], s_last[3]));
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
             lo[c] = fminf(fminf(s_box[0][c], s_box[1][c]), fminf(s_box[2][c], s_box[3][c]));
@@ -339,11 +370,11 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     }
     const bool use_fract = fract_mode > 0 || (fract_mode == 0 && !wg_safe);
     if (use_fract)
-        we_body<KT, SPLIT, true, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
-                                 i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
+        we_body<KT, SPLIT, true, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, j_end, K, zN, tid, lane, wave,
+                                 i, i_in, i_valid, xi, yi, zi, k0, wave_active, kr);
     else
-        we_body<KT, SPLIT, false, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, K, zN, tid, lane, wave,
-                                  i, i_in, i_valid, any_valid, xi, yi, zi, k0, wave_active, kr);
+        we_body<KT, SPLIT, false, MAG>(s_keys, s_wcount, s_red, cz, mz, layout, out, cos_sums, sin_sums, N, j_end, K, zN, tid, lane, wave,
+                                  i, i_in, i_valid, xi, yi, zi, k0, wave_active, kr);
 }
 
 
