@@ -105,6 +105,39 @@ def test_cfg4_shape_embedding_and_first_attention_on_sampled_rows(gpu):
         assert (O[~fin] == 0).all()
 
 
+def test_forward_replays_bit_equal_from_a_captured_graph(gpu):
+    """Every entry point launches on the caller's stream without allocating or synchronising, so a forward can be
+    captured into a graph.  Replays (with eager work and synchronisations between them) must reproduce the eager result."""
+    torch.manual_seed(7)
+    model = pa.ProteusEncoder(d_model=256, heads=4, layers=2, d_hidden=512).eval().to(gpu)
+    g = torch.Generator().manual_seed(7)
+    coords = torch.stack([synth.random_walk_chain(300, g) for _ in range(3)]).to(gpu)
+    tokens = torch.randint(0, 33, (3, 300), generator=g).to(gpu)
+    mask = torch.zeros(3, 300, dtype=torch.bool, device=gpu)
+    mask[1, 200:] = True
+    mask[2, 77:] = True
+    with torch.no_grad():
+        eager = model(coords, tokens, mask).clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                model(coords, tokens, mask)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(coords, tokens, mask)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            out.fill_(float("nan"))
+            model(coords, tokens, mask)                     # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out[~mask], eager[~mask])
+
+
 def test_training_step_through_both_kernels(gpu):
     # forward and backward of the whole stack on the HIP kernels (attention backward, wavenumber backward of the
     # embedding), one SGD step, and the loss goes down
