@@ -224,6 +224,11 @@ def main():
                                         "add_vector_operands": rates["add_v"], "transcendental": r_trans},
             "model_ms": t_model_ms, "frac": t_model_ms / avg_kernel_ms,
         },
+        # the same model with the vendor-derived rates instead of the measured ones: 256 CUs x 4 SIMDs x 16 lanes x
+        # 2.4 GHz for the five ordinary operations, a quarter of that for the two transcendentals
+        "vendor_rate_model": {"lane_ops_per_s": {"ordinary": 3.93e13, "transcendental": 9.83e12},
+                              "model_ms": W * (5.0 / 3.93e13 + 2.0 / 9.83e12) * 1e3,
+                              "frac": W * (5.0 / 3.93e13 + 2.0 / 9.83e12) * 1e3 / avg_kernel_ms},
     }
     pw = read_profile(PROFILE_WE)
     if "valu_insts_per_unit" in pw:
