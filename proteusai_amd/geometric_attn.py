@@ -229,11 +229,16 @@ class GeoAttention(nn.Module):
     logits are the reference module's (beta-weighted bias, [min_rbf, max_rbf]
     pair mask); otherwise beta_weights is kept only so that state dicts line up.
     min_rbf=None takes the reference module's default 0.001 (encoder.py:57) with legacy_logits and 0 without
-    (the README logits have no pair mask)."""
+    (the README logits have no pair mask).  operand_dtype=torch.float16 (legacy_logits only) runs the kernels on fp16
+    operands as the reference's do (old/old_scripts/attn/geometric_attn.py:567-569); default bf16.
+    d_model / heads must be 32, 64 or 128."""
 
     def __init__(self, d_model=512, heads=8, min_spread=2.0, min_rbf=None, max_rbf=1.00, learn_spreads=True,
-                 legacy_logits=False):
+                 legacy_logits=False, operand_dtype=None):
         super().__init__()
+        if operand_dtype not in (None, torch.bfloat16) and not legacy_logits:
+            raise NotImplementedError("fp16 operands go with legacy_logits=True; the README logits run in bf16")
+        self.operand_dtype = operand_dtype
         if min_rbf is None:
             min_rbf = 0.001 if legacy_logits else 0.0
         self.legacy_logits = legacy_logits      # True: the reference module's beta-weighted bias and pair mask
@@ -289,7 +294,8 @@ class GeoAttention(nn.Module):
         # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
         if self.legacy_logits:
             out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf,
-                                 max_rbf=self.max_rbf, check_spreads=False, token_major_out=True, out_dtype=q.dtype)
+                                 max_rbf=self.max_rbf, check_spreads=False, token_major_out=True, out_dtype=q.dtype,
+                                 operand_dtype=self.operand_dtype)
         else:
             out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False,
                                  token_major_out=True, out_dtype=q.dtype)

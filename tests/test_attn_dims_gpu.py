@@ -184,3 +184,28 @@ def test_the_reference_test_shape_at_its_own_tolerance(gpu):
         for got, want, name in ((q.grad, rounded[1], "dQ"), (k.grad, rounded[2], "dK"), (v.grad, rounded[3], "dV"),
                                 (s.grad, rounded[4], "d_spreads"), (b.grad, rounded[5], "d_betas")):
             assert torch.allclose(got.cpu(), want, atol=atol, rtol=0), f"{dtype} {name}: {(got.cpu() - want).abs().max():.3e}"
+
+
+def test_module_at_head_dimension_32_with_fp16_operands(gpu):
+    # the reference's module configuration: d_model 128, 4 heads (d_k = 32), beta-weighted logits, fp16 inside the kernel
+    torch.manual_seed(3)
+    mods = [pa.GeoAttention(d_model=128, heads=4, legacy_logits=True, operand_dtype=dt).to(gpu) for dt in (torch.float16, None)]
+    mods[1].load_state_dict(mods[0].state_dict())
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 90, 128, generator=g).to(gpu)
+    coords = torch.stack([synth.random_walk_chain(90, g) for _ in range(2)]).to(gpu)
+    mask = torch.zeros(2, 90, dtype=torch.bool, device=gpu)
+    mask[1, 60:] = True
+    outs = []
+    for m in mods:
+        xi = x.clone().requires_grad_(True)
+        y = m(xi, xi, xi, coords, mask)
+        y[~mask].square().mean().backward()
+        assert torch.isfinite(y[~mask]).all() and torch.isfinite(xi.grad).all()
+        assert m.spread_weights.grad.abs().sum() > 0 and m.beta_weights.grad.abs().sum() > 0
+        outs.append((y.detach(), xi.grad))
+    # the two operand types agree to their rounding
+    assert (outs[0][0] - outs[1][0])[~mask].abs().max() <= 2e-2
+    assert rel_l2(outs[0][1].cpu().numpy(), outs[1][1].cpu().numpy()) <= 3e-2
+    with pytest.raises(NotImplementedError):
+        pa.GeoAttention(d_model=128, heads=4, operand_dtype=torch.float16)
