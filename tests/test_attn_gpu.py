@@ -339,6 +339,20 @@ def test_cfg5_sampled_rows(gpu):
     assert np.abs(O1 - 1).max() < 1e-2
 
 
+def test_long_ragged_sequence_sampled_rows(gpu):
+    # N = 40003 (not a multiple of the key tile, 626 tiles, offsets beyond 5 MB per head) with tail padding, two heads,
+    # through the kernel large grids take; the last rows and the rows around the end of the unpadded part included
+    N, valid = 40003, 39000
+    wc, _ = synth.we_inputs(65536, seed=8, compact=True)
+    Q, K, V, coords, sigma, _ = synth.attn_inputs(1, 2, N, 64, seed=8, coords=wc[:, :N].contiguous())
+    mask = (torch.arange(N) >= valid)[None, :]
+    got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
+    rows = np.unique(np.concatenate([np.random.default_rng(8).choice(valid, 24, replace=False),
+                                     [0, 63, 64, valid - 1, valid, N - 1]])).astype(np.int32)
+    check(got, Q, K, V, coords, sigma, mask, rows=rows, what="N=40003")
+    assert (got[0][:, :, valid:] == 0).all() and np.isneginf(got[1][:, :, valid:]).all()
+
+
 def test_legacy_logits(gpu):
     # the reference kernel's own logits S + beta*rbf_norm*|S| with its [min_rbf, max_rbf] pair mask
     # (old/old_scripts/attn/geometric_attn.py:193-201), against the restated torch_attn oracle
