@@ -238,6 +238,47 @@ def geo_attn_scalar_grad_mass(Q, K, V, dO, coords, sigma, key_padding_mask=None,
     return mass_sigma, (spread * w_beta.abs()).sum(dim=(0, 2, 3)), total_sigma, (signed * w_beta).sum(dim=(0, 2, 3))
 
 
+def geo_attn_backward_tiled_torch(Q, K, V, dO, coords, sigma, key_padding_mask=None, row_chunk=2048, dtype=torch.float64):
+    """Gradients of the README-logit attention at sizes where the dense N x N statement does not fit: the hand-derived
+    formulas of old/old_scripts/attn/geometric_attn.py:448-505 with t = S (1 + rbf), evaluated over chunks of query rows
+        P = softmax(t); dP = dO V^T; D = sum_j P dP; dt = P (dP - D); dS = dt (1 + rbf)
+        dQ = dS K / sqrt(d); dK = dS^T Q / sqrt(d); dV = P^T dO; d sigma_h = sum dt S rbf d^2 / sigma_h^3
+    Not a second source of truth: tests/test_oracle_attn.py pins it to torch.autograd through
+    geo_attn_autograd_torch.  Also returns the pair mass of d sigma (see geo_attn_scalar_grad_mass).
+
+    Q, K, V, dO [Z,H,N,d]; coords [Z,N,3]; sigma [H]; mask [Z,N] bool.  Returns (dQ, dK, dV, d_sigma [H], mass_sigma [H])."""
+    Q, K, V, dO = Q.to(dtype), K.to(dtype), V.to(dtype), dO.to(dtype)
+    coords, sigma = coords.to(dtype), sigma.to(dtype)
+    Z, H, N, d = Q.shape
+    mask = torch.zeros(Z, N, dtype=torch.bool) if key_padding_mask is None else key_padding_mask.bool()
+    dQ, dK, dV = torch.zeros_like(Q), torch.zeros_like(K), torch.zeros_like(V)
+    d_sigma, mass = torch.zeros(H, dtype=dtype), torch.zeros(H, dtype=dtype)
+    isd = 1.0 / math.sqrt(d)
+    sg = sigma[:, None, None]
+    for z in range(Z):
+        for a in range(0, N, row_chunk):
+            r = slice(a, min(a + row_chunk, N))
+            S = torch.matmul(Q[z][:, r], K[z].transpose(1, 2)) * isd                        # H x r x N
+            d2 = torch.sum((coords[z][r][:, None, :] - coords[z][None, :, :]) ** 2, dim=2)[None]
+            rbf = torch.exp(-d2 / (2 * sg ** 2))
+            am = (mask[z][r][:, None] | mask[z][None, :])[None].expand_as(S)
+            T = torch.where(am, torch.full_like(S, float("-inf")), S * (1 + rbf))
+            row_any = (~am).any(dim=-1, keepdim=True)
+            T = torch.where(row_any, T, torch.zeros_like(T))
+            P = torch.softmax(T, dim=-1) * row_any.to(dtype)
+            dP = torch.matmul(dO[z][:, r], V[z].transpose(1, 2))
+            Dr = (P * dP).sum(dim=-1, keepdim=True)
+            dT = P * (dP - Dr)
+            dS = dT * (1 + rbf)
+            dQ[z][:, r] = torch.matmul(dS, K[z]) * isd
+            dK[z] += torch.matmul(dS.transpose(1, 2), Q[z][:, r]) * isd
+            dV[z] += torch.matmul(P.transpose(1, 2), dO[z][:, r])
+            w = S * rbf * d2 / sg ** 3
+            d_sigma += (dT * w).sum(dim=(1, 2))
+            mass += (P * (dP.abs() + Dr.abs()) * w.abs()).sum(dim=(1, 2))
+    return dQ, dK, dV, d_sigma, mass
+
+
 def encoder_forward_torch(params, min_spread, coords, tokens, mask, attention=None):
     """The encoder stack in fp32 on the CPU with the oracles in place of the kernels: WE(coords) + embedding[tokens],
     then per layer geometric multi-head attention on the projections of x (per-head [d_model, d_k] weights and

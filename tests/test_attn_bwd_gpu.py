@@ -231,6 +231,27 @@ def test_cfg3_shape_sampled(gpu):
     compare(gpu_grads(gpu, Q, K, V, dO, coords, sigma, None), reference_grads(Q, K, V, dO, coords, sigma, None), None, "N=2048")
 
 
+def test_full_length_sequence_every_gradient(gpu):
+    # N = 16384 (the benchmark's sequence length: 256 tiles of streamed tokens per workgroup, both stages of the
+    # direct-to-LDS staging reused 128 times) on the compacted chain, the narrowest and the widest head of the
+    # benchmark's sigma range, against the tiled statement of the gradient formulas (pinned to torch.autograd on the CPU
+    # in tests/test_oracle_attn.py; fp32 here, which differs from fp64 by 4e-7 in relative L2 at this size).
+    wc, _ = synth.we_inputs(65536, seed=5, compact=True)
+    Z, H, N = 1, 2, 16384
+    Q, K, V, coords, sigma, _ = synth.attn_inputs(Z, H, N, 64, 5, coords=wc[:, :N].contiguous())
+    g = torch.Generator().manual_seed(5)
+    dO = (torch.randn(Z, H, N, 64, generator=g) / 8).bfloat16()
+    got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, None)
+    rQ, rK, rV, rs, mass = torch_oracle.geo_attn_backward_tiled_torch(Q, K, V, dO, coords, sigma, None, row_chunk=1024,
+                                                                      dtype=torch.float32)
+    for gg, rr, name in zip(got[:3], (rQ, rK, rV), ("dQ", "dK", "dV")):
+        assert torch.isfinite(gg).all(), f"N=16384 {name}: non-finite"
+        e = rel_l2(gg.numpy(), rr.numpy())
+        assert e <= REL_L2_TOL, f"N=16384 {name}: rel-L2 {e:.3e}"
+    err = (got[3].double() - rs.double()).abs()
+    assert (err <= SCALAR_TOL * mass.double()).all(), f"N=16384 d_sigma: error / pair mass {(err / mass.double()).max():.3e}"
+
+
 def test_module_trains(gpu):
     torch.manual_seed(0)
     m = pa.GeoAttention(d_model=128, heads=2).to(gpu)

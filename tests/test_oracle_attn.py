@@ -210,3 +210,28 @@ def test_per_query_sigma_and_beta_split_the_per_head_gradients():
             assert (m_b >= b_rows.grad.abs().sum(dim=(0, 2)) * (1 - 1e-12)).all()
         else:
             assert m_b is None and t_b is None
+
+
+def test_tiled_backward_equals_autograd():
+    """The chunked hand-derived gradients (used where N x N does not fit) against torch.autograd through the dense
+    differentiable statement: masks, an empty batch item but for one token, chunks that do not divide N."""
+    g = torch.Generator().manual_seed(13)
+    Z, H, N = 2, 3, 53
+    Q, K, V, dO = (torch.randn(Z, H, N, 64, generator=g, dtype=torch.float64) for _ in range(4))
+    coords = torch.cumsum(torch.randn(Z, N, 3, generator=g, dtype=torch.float64) * 2.2, dim=1)
+    sigma = torch.tensor([2.0, 5.0, 11.0], dtype=torch.float64)
+    mask = torch.rand(Z, N, generator=g) < 0.25
+    mask[1] = True
+    mask[1, 7] = False
+    q, k, v = (t.clone().requires_grad_(True) for t in (Q, K, V))
+    s = sigma.clone().requires_grad_(True)
+    torch_oracle.geo_attn_autograd_torch(q, k, v, coords, s, mask).backward(dO)
+    for chunk in (7, 16, 53, 2048):
+        dQ, dK, dV, ds, mass = torch_oracle.geo_attn_backward_tiled_torch(Q, K, V, dO, coords, sigma, mask, row_chunk=chunk)
+        torch.testing.assert_close(dQ, q.grad, rtol=1e-10, atol=1e-12)
+        torch.testing.assert_close(dK, k.grad, rtol=1e-10, atol=1e-12)
+        torch.testing.assert_close(dV, v.grad, rtol=1e-10, atol=1e-12)
+        torch.testing.assert_close(ds, s.grad, rtol=1e-9, atol=1e-12)
+        m_ref, _, t_ref, _ = torch_oracle.geo_attn_scalar_grad_mass(Q, K, V, dO, coords, sigma, mask)
+        torch.testing.assert_close(mass, m_ref, rtol=1e-10, atol=1e-14)
+        torch.testing.assert_close(ds, t_ref, rtol=1e-9, atol=1e-12)
