@@ -123,7 +123,7 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
 }
 
 // d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
-// the software-pipelined kernel runs (automatically for grids of more than 256 workgroups, or when the tuning asks).
+// the software-pipelined kernel runs (automatically for grids of at least 256 workgroups = one per CU, or when the tuning asks).
 int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords,
                 const float* sigma, const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
@@ -135,7 +135,7 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
         return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 0 : tuning,
                                                beta, min_rbf, max_rbf, gs, st);
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
-    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 > 256)))
+    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 256)))
         return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
     return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
