@@ -495,6 +495,32 @@ def main():
             "ms": e0.elapsed_time(e1) / 10, "valid_tokens": int(lens.sum()),
             "tokens_per_s": float(lens.sum()) / (e0.elapsed_time(e1) / 10 * 1e-3),
         }
+        # the same forward captured into a HIP graph and replayed: what the launches cost goes away
+        with torch.no_grad():
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                model(ecoords, etokens, emask)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                graph_out = model(ecoords, etokens, emask)
+            torch.cuda.synchronize()
+            eager_out = model(ecoords, etokens, emask)
+            graph.replay()
+            torch.cuda.synchronize()
+            same = bool(torch.equal(graph_out[~emask], eager_out[~emask]))
+            settle(torch, graph.replay)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+        result["encoder_forward"]["ms_graph_replay"] = e0.elapsed_time(e1) / 10
+        result["encoder_forward"]["graph_replay_equals_eager"] = same
+        del graph, graph_out
         if not args.no_cpu:
             with torch.no_grad():
                 dt, runs = cpu_timed(lambda: torch_oracle.encoder_forward_torch(state, min_spread, ecoords_h, etokens_h, emask_h), 20.0, 3)
