@@ -43,6 +43,7 @@
 
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include <type_traits>
 #include "proteus_hip.h"
@@ -110,9 +111,17 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
                      const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, bool take_all,
                      const GaStrides& gs, hipStream_t st)
 {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)GA_PIPE_LDS);
-    if (attr != hipSuccess) return (int)attr;
+    // more than 64 KB of dynamic LDS must be allowed once per device (remembered for the first 64 devices)
+    static std::atomic<unsigned long long> allowed{0ull};
+    int dev = 0;
+    const hipError_t got = hipGetDevice(&dev);
+    if (got != hipSuccess) return (int)got;
+    if (dev < 0 || dev >= 64 || !((allowed.load(std::memory_order_relaxed) >> dev) & 1ull)) {
+        const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)GA_PIPE_LDS);
+        if (attr != hipSuccess) return (int)attr;
+        if (dev >= 0 && dev < 64) allowed.fetch_or(1ull << dev, std::memory_order_relaxed);
+    }
     constexpr int BM = GA_WAVES * 64;
     const int n_qtiles = (N + BM - 1) / BM;
     const int ZH = Z * H;
