@@ -202,6 +202,43 @@ def test_pairs_on_the_rbf_thresholds_are_in_range_in_both_passes_or_in_neither(g
             assert ((col_sums - rows_with_a_pair).abs() <= 1e-2 * rows_with_a_pair).all(), (kind, float(thr), col_sums, rows_with_a_pair)
 
 
+def test_tiles_skipped_below_min_rbf_hold_no_pair_in_range(gpu):
+    """With a lower rbf bound the kernels skip key tiles (forward) and blocks (backward) that lie out of reach of a wave's
+    tokens, where every pair is masked.  Here the tokens of the first tile sit in a tight cluster and the others on
+    shells around it whose rbf against the cluster is min_rbf times 0.9, 0.99, 0.999, 1.001, 1.01 and 1.1 (shell by
+    shell, so whole tiles are just out of or just in range): the logsumexp of the cluster's queries and the dK, dV rows
+    of the shell tokens change by far more than the bar if a tile with pairs in range is dropped, or one without is kept."""
+    Z, H, N = 1, 2, 64 + 6 * 64
+    g = torch.Generator().manual_seed(29)
+    Q = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    K = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    dO = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    sigma = torch.tensor([6.0, 9.0])
+    betas = torch.tensor([0.7, -0.4])
+    lo, hi = 0.01, 1.0
+    coords = torch.zeros(Z, N, 3)
+    coords[0, :64] = torch.randn(64, 3, generator=g) * 1e-5 + torch.tensor([4.0, -2.5, 1.0])
+    for shell, f in enumerate((0.9, 0.99, 0.999, 1.001, 1.01, 1.1)):
+        r = float(np.sqrt(-2.0 * 36.0 * np.log(lo * f)))                    # rbf(r) = lo * f for head 0 (sigma 6)
+        d = torch.randn(64, 3, generator=g)
+        coords[0, 64 + 64 * shell: 128 + 64 * shell] = coords[0, :64].mean(0) + r * d / d.norm(dim=1, keepdim=True)
+    got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, None, betas, lo, hi)
+    ref = reference_grads(Q, K, V, dO, coords, sigma, None, betas, lo, hi)
+    compare(got, ref, None, "shells around min_rbf")
+    # row by row: a dropped or an extra tile changes whole rows of dK and dV
+    for gg, rr, name in zip(got[1:3], ref[1:3], ("dK", "dV")):
+        err = (gg.double() - rr).norm(dim=-1)
+        assert (err <= 2e-2 * rr.norm(dim=-1) + 2e-2 * rr.norm(dim=-1).mean()).all(), f"{name} rows: {(err / rr.norm(dim=-1).mean()).max():.3e}"
+    _, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), None, return_lse=True,
+                       betas=betas.to(gpu), min_rbf=lo, max_rbf=hi)
+    _, Lref = torch_oracle.geo_attn_legacy_torch(Q.float(), K.float(), V.float(), coords, sigma, betas, None, lo, hi, dtype=torch.float64)
+    assert (L.cpu().double() - Lref).abs().max() <= 4e-3, f"logsumexp {(L.cpu().double() - Lref).abs().max():.3e}"
+    # and the cluster's queries do see exactly the three shells in range, beside the cluster itself (head 0)
+    n_in = ((torch.cdist(coords[0, :64].double(), coords[0].double()) ** 2 / -72.0).exp() >= lo).sum(dim=1)
+    assert (n_in == 64 + 3 * 64).all()
+
+
 def test_large_logits(gpu):
     a = make(3, 1, 4, 400, qscale=2.5)
     compare(gpu_grads(gpu, *a), reference_grads(*a), None, "large logits")
