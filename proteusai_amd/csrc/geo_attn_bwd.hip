@@ -21,10 +21,9 @@
 // token: S = other . own^T and dP likewise on v_mfma_f32_32x32x16_bf16 with the own side held in registers
 // as the B operand for the whole kernel.  P and dS are, after bf16 conversion, directly the B operands of
 // the accumulating products (dV^T += dO^T P, dK^T += Q^T dS; dQ^T += K^T dS) whose A operands are the
-// streamed tiles transposed, read in the accumulator's row order: at d = 64 the tiles travel global -> LDS
-// directly and are transposed by the LDS read (ds_read_b64_tr_b16); at d = 32 and 128 a second, transposed
-// copy is staged through registers.  No atomics except the one per-wave add into d sigma / d beta; dQ, dK,
-// dV are deterministic.
+// streamed tiles transposed, read in the accumulator's row order: the tiles travel global -> LDS directly
+// and are transposed by the LDS read (ds_read_b64_tr_b16).  No atomics except the one per-wave add into
+// d sigma / d beta; dQ, dK, dV are deterministic.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
