@@ -71,4 +71,20 @@ template <> struct HeadDim<32>  { static constexpr float QS = 0.25f,  RHO = 0.70
 template <> struct HeadDim<64>  { static constexpr float QS = 0.125f, RHO = 1.0f,                 INV_SQRT = 0.125f; };
 template <> struct HeadDim<128> { static constexpr float QS = 0.125f, RHO = 0.70710678118654752f, INV_SQRT = 0.08838834764831845f; };
 
+// XOR swizzle of the 16-byte chunks of a row-major LDS tile of 16-bit elements with rows of 2 D bytes (chunk c of
+// row r sits at slot c ^ tile_swizzle<D>(r)), under which both kinds of reads are free of bank conflicts (64 banks of
+// 4 bytes):
+//  * 16-byte fragment reads: 16 lanes read one chunk of 16 consecutive rows;
+//  * transposing reads (ds_read_b64_tr_b16): 16 lanes read 32 bytes (an even chunk and the next) of four consecutive
+//    rows, aligned to four.
+// d = 32 (64-byte rows: rows r, r+4, r+8, r+12 share banks): (r >> 2) & 3.
+// d = 64 (128-byte rows: the even and the odd rows each share banks): the 8 even and the 8 odd rows of 16 consecutive
+//   ones get 8 different values, and rows r, r + 2 of an aligned group of four differ in bits 1..2.
+// d = 128 (256-byte rows: all rows share banks): a permutation of r & 15 whose upper three bits differ among four
+//   consecutive rows.
+template <int D> __device__ __forceinline__ int tile_swizzle(int r);
+template <> __device__ __forceinline__ int tile_swizzle<32>(int r)  { return (r >> 2) & 3; }
+template <> __device__ __forceinline__ int tile_swizzle<64>(int r)  { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
+template <> __device__ __forceinline__ int tile_swizzle<128>(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
 }  // namespace proteus_ops
