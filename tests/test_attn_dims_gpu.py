@@ -67,6 +67,33 @@ def test_forward_readme_logits(gpu, d, N):
         check_forward(O, L, Q, K, V, coords, sigma, mask, None, 0.0, 1.0, LSE_TOL_BF16, f"d={d} N={N} tuning={tuning}")
 
 
+@pytest.mark.parametrize("d", [32, 128])
+def test_forward_long_ragged_sequence_sampled_rows(gpu, d):
+    # N = 5003 (79 tiles, the last one ragged), tail padding, both kinds of logits: the two LDS stages of the directly
+    # loaded tiles are reused 39 times; sampled query rows against the torch oracle
+    Z, H, N = 1, 2, 5003
+    Q, K, V, _, coords, sigma, _ = make(900 + d, Z, H, N, d, torch.bfloat16)
+    mask = torch.zeros(Z, N, dtype=torch.bool)
+    mask[0, 4700:] = True
+    rows = np.sort(np.random.default_rng(d).choice(4700, 48, replace=False))
+    betas = torch.tensor([0.6, -0.3])
+    for bt, lo, hi in ((None, 0.0, 1.0), (betas, 0.01, 0.97)):
+        O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), return_lse=True,
+                           betas=None if bt is None else bt.to(gpu), min_rbf=lo, max_rbf=hi)
+        O, L = O.cpu().double(), L.cpu().double()
+        assert torch.isfinite(O).all() and (O[0, :, 4700:] == 0).all() and torch.isneginf(L[0, :, 4700:]).all()
+        if bt is None:
+            Or, Lr = torch_oracle.geo_attn_torch(Q.float(), K.float(), V.float(), coords, sigma, mask, rows=rows, dtype=torch.float64)
+        else:
+            # (the dense legacy statement has no row subset: two heads of 5003^2 pairs in fp64 fit)
+            Or, Lr = torch_oracle.geo_attn_legacy_torch(Q.float(), K.float(), V.float(), coords, sigma, bt, mask, lo, hi, dtype=torch.float64)
+            Or, Lr = Or[:, :, rows], Lr[:, :, rows]
+        fin = torch.isfinite(Lr)
+        assert (torch.isfinite(L[:, :, rows]) == fin).all()
+        assert (O[:, :, rows] - Or).abs().max() <= MAX_ABS_TOL, f"d={d} legacy={bt is not None}: O {(O[:, :, rows] - Or).abs().max():.3e}"
+        assert (L[:, :, rows][fin] - Lr[fin]).abs().max() <= LSE_TOL_BF16, f"d={d} legacy={bt is not None}: L {(L[:, :, rows][fin] - Lr[fin]).abs().max():.3e}"
+
+
 @pytest.mark.parametrize("d", [32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_forward_legacy_logits(gpu, d, dtype):
