@@ -461,7 +461,34 @@ def main():
                              "unit": "TFLOP/s", "frac": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
                              "traffic": b_traffic, "traffic_source": b_traffic_src},
             }
-            del dOb, Dv, dQ_, dK_, dV_
+            # ---- the reference kernel's own logits (beta-weighted bias, pair mask) at its module's default rbf range:
+            #      key tiles whose pairs are all below min_rbf are skipped ----
+            bet = torch.full((8,), 0.5, device=dev)
+            dbt = torch.zeros(8, device=dev)
+            lo_rbf, hi_rbf = 0.001, 1.0
+
+            def legacy_fwd():
+                rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), acd.data_ptr(), sg.data_ptr(), bet.data_ptr(),
+                                                     None, O.data_ptr(), L.data_ptr(), 1, 8, 16384, 64, lo_rbf, hi_rbf,
+                                                     _lib.OPERAND_BF16, 0, stream)
+                if rc != 0:
+                    _lib.check(rc, "proteus_geo_attn_legacy_fwd")
+
+            def legacy_bwd():
+                rc = lib.proteus_geo_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dOb.data_ptr(), acd.data_ptr(), sg.data_ptr(),
+                                              bet.data_ptr(), None, L.data_ptr(), Dv.data_ptr(), dQ_.data_ptr(), dK_.data_ptr(), dV_.data_ptr(),
+                                              dsg.data_ptr(), dbt.data_ptr(), 1, 8, 16384, 64, lo_rbf, hi_rbf, _lib.OPERAND_BF16, stream)
+                if rc != 0:
+                    _lib.check(rc, "proteus_geo_attn_bwd")
+            lf_ms, _ = time_launches(torch, legacy_fwd, 10)
+            Dv = (O * dOb.float()).sum(-1).contiguous()
+            lb_ms, _ = time_launches(torch, legacy_bwd, 5)
+            result["geo_attn_reference_logits"] = {
+                "workload": "the same shape with the reference kernel's logits S + beta*rbf_norm*|S| and pair mask, beta 0.5, "
+                            "rbf range [0.001, 1] (the reference module's default), bf16 operands",
+                "forward_ms": lf_ms, "backward_ms": lb_ms,
+                "note": "pairs below min_rbf are masked, so tiles out of reach are skipped: the time depends on sigma"}
+            del dOb, Dv, dQ_, dK_, dV_, bet, dbt
         del q, k, v, O, L
 
     # ---------------- encoder forward, B=8, N=1024, 4 layers, bf16 weights, fp32 WE (configs[3]) ----------------
