@@ -22,6 +22,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "proteus_hip.h"
 
 namespace {
@@ -29,6 +30,9 @@ namespace {
 constexpr int WA_WAVES   = 4;
 constexpr int WA_THREADS = WA_WAVES * 64;
 constexpr int WA_JB      = 256;   // sources staged per LDS block (one per thread)
+// v_sin / v_cos take revolutions and are exact-period up to 256 of them: phases that provably stay below this need no
+// explicit reduction (v_fract)
+constexpr float WA_MAX_REV = 250.0f;
 
 __device__ __forceinline__ float sgpr(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
@@ -47,6 +51,8 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     __shared__ float4 s_ka[WA_JB + WA_WAVES];    // source positions   (padding: the loop reads one step ahead)
     __shared__ float4 s_kb[WA_JB + WA_WAVES];    // source C-beta vectors
     __shared__ int    s_wcount[WA_WAVES];
+    __shared__ float  s_box[WA_WAVES][8];        // per wave: bounding box of the unpadded positions, largest |b|^2
+    __shared__ int    s_last[WA_WAVES];
     __shared__ float  s_red[SPLIT ? (WA_WAVES - 1) * (6 * KT + 1) * 64 : 1];
 
     const int tid  = threadIdx.x;
@@ -82,13 +88,84 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
         ck[t] = sgpr((float)((double)w * (double)c * 0.15915494309189533577));
     }
 
+    int  j_end = 0;
+    bool use_fract = true;
+    if (any_valid) {
+        // ---- Can any phase of this workgroup leave the range v_sin / v_cos accept?  |phase| <= r kr + |A| ck with
+        // r <= the distance from the observer to the farthest corner of the box of the unpadded positions and
+        // |A| = |b_j . R| / r <= |b_j|.  One pass over the batch item (a few loads per thread) finds the box, the
+        // largest |b_j| and where the unpadded sources end (the blocks behind that are never staged). ----
+        {
+            float lo[3] = {3.0e38f, 3.0e38f, 3.0e38f}, hi[3] = {-3.0e38f, -3.0e38f, -3.0e38f}, b2max = 0.f;
+            int last = 0;
+            for (int j = tid; j < N; j += WA_THREADS) {
+                if (mz && mz[j]) continue;
+                last = j + 1;
+                float p[3], q[3];
+                if (layout == PROTEUS_COORDS_SOA) {
+                    p[0] = az[j]; p[1] = az[(size_t)N + j]; p[2] = az[2 * (size_t)N + j];
+                    q[0] = bz[j]; q[1] = bz[(size_t)N + j]; q[2] = bz[2 * (size_t)N + j];
+                } else {
+                    p[0] = az[3 * (size_t)j]; p[1] = az[3 * (size_t)j + 1]; p[2] = az[3 * (size_t)j + 2];
+                    q[0] = bz[3 * (size_t)j]; q[1] = bz[3 * (size_t)j + 1]; q[2] = bz[3 * (size_t)j + 2];
+                }
+#pragma unroll
+                for (int c = 0; c < 3; ++c) { lo[c] = fminf(lo[c], p[c]); hi[c] = fmaxf(hi[c], p[c]); }
+                const float b2 = q[0] * q[0] + q[1] * q[1] + q[2] * q[2];
+                b2max = (b2 <= b2max) ? b2max : b2;          // (a NaN sticks: the reducing path is taken)
+            }
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                for (int o = 32; o > 0; o >>= 1) { lo[c] = fminf(lo[c], __shfl_xor(lo[c], o)); hi[c] = fmaxf(hi[c], __shfl_xor(hi[c], o)); }
+            for (int o = 32; o > 0; o >>= 1) {
+                last = max(last, __shfl_xor(last, o));
+                const float other = __shfl_xor(b2max, o);
+                b2max = (other <= b2max) ? b2max : other;
+            }
+            if (lane == 0) {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) { s_box[wave][c] = lo[c]; s_box[wave][3 + c] = hi[c]; }
+                s_box[wave][6] = b2max;
+                s_last[wave] = last;
+            }
+            __syncthreads();
+            j_end = max(max(s_last[0], s_last[1]), max(s_last[2], s_last[3]));
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                lo[c] = fminf(fminf(s_box[0][c], s_box[1][c]), fminf(s_box[2][c], s_box[3][c]));
+                hi[c] = fmaxf(fmaxf(s_box[0][3 + c], s_box[1][3 + c]), fmaxf(s_box[2][3 + c], s_box[3][3 + c]));
+            }
+            b2max = s_box[0][6];
+#pragma unroll
+            for (int w = 1; w < WA_WAVES; ++w) b2max = (s_box[w][6] <= b2max) ? b2max : s_box[w][6];
+            float kr_max = 0.f, ck_max = 0.f;
+#pragma unroll
+            for (int t = 0; t < KT; ++t) { kr_max = fmaxf(kr_max, fabsf(kr[t])); ck_max = fmaxf(ck_max, fabsf(ck[t])); }
+            const float fx = fmaxf(fabsf(xi - lo[0]), fabsf(xi - hi[0]));
+            const float fy = fmaxf(fabsf(yi - lo[1]), fabsf(yi - hi[1]));
+            const float fz = fmaxf(fabsf(zi - lo[2]), fabsf(zi - hi[2]));
+            const float rfar = __builtin_sqrtf(fx * fx + fy * fy + fz * fz);
+            // NaN-safe: anything that is not provably below the limit takes the reducing path
+            // (a padded observer's lane, whose coordinates may hold anything, has no say)
+            const bool wave_safe = __builtin_amdgcn_ballot_w64(i_valid && !(rfar * kr_max + __builtin_sqrtf(b2max) * ck_max < WA_MAX_REV)) == 0;
+            if (lane == 0) s_wcount[wave] = wave_safe ? 1 : 0;
+            __syncthreads();
+            use_fract = (s_wcount[0] & s_wcount[1] & s_wcount[2] & s_wcount[3]) == 0;
+            __syncthreads();                       // s_wcount is reused by the staging below
+        }
+    }
+
+    // Everything from here on exists twice, with and without the explicit phase reduction, as two instances of one
+    // generic lambda: the running sums live inside it, so the two sets are never alive together.
+    auto rest = [&](auto fract_c) {
+    constexpr bool FRACT = decltype(fract_c)::value;
     float s1[KT], s2[KT], s3[KT], s4[KT], s5[KT], s6[KT];
 #pragma unroll
     for (int t = 0; t < KT; ++t) { s1[t] = 0.f; s2[t] = 0.f; s3[t] = 0.f; s4[t] = 0.f; s5[t] = 0.f; s6[t] = 0.f; }
     float nzero = 0.f;
 
     if (any_valid) {
-        for (int jb = 0; jb < N; jb += WA_JB) {
+        for (int jb = 0; jb < j_end; jb += WA_JB) {
             // -- stage one block of sources, keeping only the unpadded ones --
             const int  j    = jb + tid;
             const bool j_in = j < N;
@@ -121,36 +198,39 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
             if (!wave_active) continue;
 
             // -- stream the staged sources --
-            const int first = SPLIT ? wave : 0;
-            const int step  = SPLIT ? WA_WAVES : 1;
-            float4 anext = s_ka[first], bnext = s_kb[first];
+            {
+                const int first = SPLIT ? wave : 0;
+                const int step  = SPLIT ? WA_WAVES : 1;
+                float4 anext = s_ka[first], bnext = s_kb[first];
 #pragma unroll 1
-            for (int jj = first; jj < nk; jj += step) {
-                const float4 a = anext, b = bnext;
-                anext = s_ka[jj + step];
-                bnext = s_kb[jj + step];
-                const float dx = xi - a.x, dy = yi - a.y, dz = zi - a.z;
-                const float r2 = dx * dx + dy * dy + dz * dz;
-                const bool  ok = r2 != 0.0f;
-                const float inv = ok ? __builtin_amdgcn_rsqf(r2) : 0.0f;
-                // one Newton step on r = r2 * rsq(r2): r is then within 1 ulp of sqrt(r2)
-                const float r0 = r2 * inv;
-                const float e  = __builtin_fmaf(-r0, r0, r2);
-                const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
-                const float A  = inv * __builtin_fmaf(b.x, dx, __builtin_fmaf(b.y, dy, b.z * dz));
-                const float v  = inv * A;
-                nzero += ok ? 0.0f : 1.0f;
+                for (int jj = first; jj < nk; jj += step) {
+                    const float4 a = anext, b = bnext;
+                    anext = s_ka[jj + step];
+                    bnext = s_kb[jj + step];
+                    const float dx = xi - a.x, dy = yi - a.y, dz = zi - a.z;
+                    const float r2 = dx * dx + dy * dy + dz * dz;
+                    const bool  ok = r2 != 0.0f;
+                    const float inv = ok ? __builtin_amdgcn_rsqf(r2) : 0.0f;
+                    // one Newton step on r = r2 * rsq(r2): r is then within 1 ulp of sqrt(r2)
+                    const float r0 = r2 * inv;
+                    const float e  = __builtin_fmaf(-r0, r0, r2);
+                    const float r  = __builtin_fmaf(e, 0.5f * inv, r0);
+                    const float A  = inv * __builtin_fmaf(b.x, dx, __builtin_fmaf(b.y, dy, b.z * dz));
+                    const float v  = inv * A;
+                    nzero += ok ? 0.0f : 1.0f;
 #pragma unroll
-                for (int t = 0; t < KT; ++t) {
-                    const float ph = __builtin_amdgcn_fractf(__builtin_fmaf(-A, ck[t], r * kr[t]));
-                    const float s = __builtin_amdgcn_sinf(ph);
-                    const float c = __builtin_amdgcn_cosf(ph);
-                    s1[t] = __builtin_fmaf(c, inv, s1[t]);
-                    s2[t] = __builtin_fmaf(s, inv, s2[t]);
-                    s3[t] += c;
-                    s4[t] += s;
-                    s5[t] = __builtin_fmaf(c, v, s5[t]);
-                    s6[t] = __builtin_fmaf(s, v, s6[t]);
+                    for (int t = 0; t < KT; ++t) {
+                        float ph = __builtin_fmaf(-A, ck[t], r * kr[t]);
+                        if (FRACT) ph = __builtin_amdgcn_fractf(ph);
+                        const float s = __builtin_amdgcn_sinf(ph);
+                        const float c = __builtin_amdgcn_cosf(ph);
+                        s1[t] = __builtin_fmaf(c, inv, s1[t]);
+                        s2[t] = __builtin_fmaf(s, inv, s2[t]);
+                        s3[t] += c;
+                        s4[t] += s;
+                        s5[t] = __builtin_fmaf(c, v, s5[t]);
+                        s6[t] = __builtin_fmaf(s, v, s6[t]);
+                    }
                 }
             }
         }
@@ -226,6 +306,8 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
             }
         }
     }
+    };
+    if (use_fract) rest(std::true_type{}); else rest(std::false_type{});
 }
 
 struct WaVariant { const char* name; int kt; bool split; };

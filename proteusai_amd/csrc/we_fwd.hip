@@ -363,7 +363,8 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
         const float fz = fmaxf(fabsf(zi - lo[2]), fabsf(zi - hi[2]));
         const float rfar = __builtin_sqrtf(fx * fx + fy * fy + fz * fz);
         // NaN-safe: anything that is not provably below the limit takes the reducing path
-        const bool wave_safe = __builtin_amdgcn_ballot_w64(!(rfar * kr_max < WE_MAX_REV)) == 0;
+        // (a padded observer's lane, whose coordinates may hold anything, has no say)
+        const bool wave_safe = __builtin_amdgcn_ballot_w64(i_valid && !(rfar * kr_max < WE_MAX_REV)) == 0;
         if (lane == 0) s_wcount[wave] = wave_safe ? 1 : 0;
         __syncthreads();
         wg_safe = (s_wcount[0] & s_wcount[1] & s_wcount[2] & s_wcount[3]) != 0;
