@@ -312,6 +312,14 @@ def main():
                                                   "add_vector_operands": 2, "transcendental": 2},
                             "model_ms": x_model_ms, "frac": x_model_ms / x_ms},
         }
+
+        def aniso_lean_step():
+            rc = lib.proteus_we_aniso_fwd(c.data_ptr(), cbv.data_ptr(), _lib.COORDS_AOS, cbm.data_ptr(), w.data_ptr(), None,
+                                          ao[0].data_ptr(), None, None, Z, N, K, 0, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_we_aniso_fwd")
+        xl_ms, _ = time_launches(torch, aniso_lean_step, max(5, args.steps // 2), 0.0)
+        result["we_aniso"]["ms_embedding_only"] = xl_ms           # d_cb = d_k = NULL: two running sums per wavenumber instead of six
         del ao
 
     # ---------------- configs[0]: WE forward B=1, N=512 (the reference's CPU-runnable case) ----------------

@@ -146,7 +146,8 @@ int proteus_we_legacy_fwd(const float* coords, int coords_layout,
  *                     (positions; per-token C-beta direction vectors)
  *   cb_magnitudes, wavenumbers  [K] f32
  *   mask              [Z,N] u8, non-zero = padded; may be NULL
- *   out, d_cb, d_k    [Z,N,2K] f32, 16-byte aligned
+ *   out, d_cb, d_k    [Z,N,2K] f32, 16-byte aligned.  d_cb and d_k may both be NULL (not one of them): then only
+ *                     the embedding is computed, with two running sums per wavenumber instead of six.
  */
 int proteus_we_aniso_fwd(const float* coordsA, const float* coordsB, int coords_layout,
                          const float* cb_magnitudes, const float* wavenumbers, const uint8_t* mask,

@@ -40,7 +40,8 @@ __device__ __forceinline__ float sgpr(float v) {
 
 // KT     wavenumbers per wave (6*KT accumulators per lane)
 // SPLIT  the four waves share one wavenumber tile and split the staged sources; partial sums meet in LDS
-template <int KT, bool SPLIT>
+// GRADS  false: only the embedding is wanted (d_cb = d_k = NULL): two sums per wavenumber instead of six
+template <int KT, bool SPLIT, bool GRADS>
 __global__ __launch_bounds__(WA_THREADS)
 void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restrict__ coordsB, const int layout,
                          const float* __restrict__ cb_magnitudes, const float* __restrict__ wavenumbers,
@@ -53,7 +54,8 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     __shared__ int    s_wcount[WA_WAVES];
     __shared__ float  s_box[WA_WAVES][8];        // per wave: bounding box of the unpadded positions, largest |b|^2
     __shared__ int    s_last[WA_WAVES];
-    __shared__ float  s_red[SPLIT ? (WA_WAVES - 1) * (6 * KT + 1) * 64 : 1];
+    constexpr int NS = GRADS ? 6 : 2;            // running sums per wavenumber
+    __shared__ float  s_red[SPLIT ? (WA_WAVES - 1) * (NS * KT + 1) * 64 : 1];
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -226,10 +228,12 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
                         const float c = __builtin_amdgcn_cosf(ph);
                         s1[t] = __builtin_fmaf(c, inv, s1[t]);
                         s2[t] = __builtin_fmaf(s, inv, s2[t]);
-                        s3[t] += c;
-                        s4[t] += s;
-                        s5[t] = __builtin_fmaf(c, v, s5[t]);
-                        s6[t] = __builtin_fmaf(s, v, s6[t]);
+                        if (GRADS) {
+                            s3[t] += c;
+                            s4[t] += s;
+                            s5[t] = __builtin_fmaf(c, v, s5[t]);
+                            s6[t] = __builtin_fmaf(s, v, s6[t]);
+                        }
                     }
                 }
             }
@@ -240,25 +244,29 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
         // ---- the four waves' partial sums meet in LDS; wave 0 writes the rows ----
         __syncthreads();
         if (wave > 0) {
-            float* q = s_red + (size_t)(wave - 1) * (6 * KT + 1) * 64 + lane;
+            float* q = s_red + (size_t)(wave - 1) * (NS * KT + 1) * 64 + lane;
 #pragma unroll
             for (int t = 0; t < KT; ++t) {
-                q[(6 * t + 0) * 64] = s1[t]; q[(6 * t + 1) * 64] = s2[t]; q[(6 * t + 2) * 64] = s3[t];
-                q[(6 * t + 3) * 64] = s4[t]; q[(6 * t + 4) * 64] = s5[t]; q[(6 * t + 5) * 64] = s6[t];
+                q[(NS * t + 0) * 64] = s1[t]; q[(NS * t + 1) * 64] = s2[t];
+                if (GRADS) {
+                    q[(NS * t + 2) * 64] = s3[t]; q[(NS * t + 3) * 64] = s4[t]; q[(NS * t + 4) * 64] = s5[t]; q[(NS * t + 5) * 64] = s6[t];
+                }
             }
-            q[6 * KT * 64] = nzero;
+            q[NS * KT * 64] = nzero;
         }
         __syncthreads();
         if (wave > 0) return;
 #pragma unroll 1
         for (int w = 0; w < WA_WAVES - 1; ++w) {
-            const float* q = s_red + (size_t)w * (6 * KT + 1) * 64 + lane;
+            const float* q = s_red + (size_t)w * (NS * KT + 1) * 64 + lane;
 #pragma unroll
             for (int t = 0; t < KT; ++t) {
-                s1[t] += q[(6 * t + 0) * 64]; s2[t] += q[(6 * t + 1) * 64]; s3[t] += q[(6 * t + 2) * 64];
-                s4[t] += q[(6 * t + 3) * 64]; s5[t] += q[(6 * t + 4) * 64]; s6[t] += q[(6 * t + 5) * 64];
+                s1[t] += q[(NS * t + 0) * 64]; s2[t] += q[(NS * t + 1) * 64];
+                if (GRADS) {
+                    s3[t] += q[(NS * t + 2) * 64]; s4[t] += q[(NS * t + 3) * 64]; s5[t] += q[(NS * t + 4) * 64]; s6[t] += q[(NS * t + 5) * 64];
+                }
             }
-            nzero += q[6 * KT * 64];
+            nzero += q[NS * KT * 64];
         }
     }
 
@@ -267,8 +275,8 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     // ---- epilogue: each lane writes its own rows ----
     const size_t row = (zN + (size_t)i) * (size_t)(2 * K) + 2 * (size_t)k0;
     float* po = out  + row;
-    float* pc = d_cb + row;
-    float* pk = d_k  + row;
+    float* pc = GRADS ? d_cb + row : nullptr;
+    float* pk = GRADS ? d_k  + row : nullptr;
     const bool vec = (k0 + KT <= K) && ((K & 1) == 0) && ((KT & 1) == 0);   // rows and tile start 16-byte aligned
     // The scales are read again here rather than kept from the prologue: held across the main loop they
     // would take 2*KT scalar registers the loop needs for kr[] and ck[].
@@ -293,15 +301,19 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
         }
         if (vec) {
             *reinterpret_cast<float4*>(po + 2 * t) = make_float4(o[0], o[1], o[2], o[3]);
-            *reinterpret_cast<float4*>(pc + 2 * t) = make_float4(g[0], g[1], g[2], g[3]);
-            *reinterpret_cast<float4*>(pk + 2 * t) = make_float4(h[0], h[1], h[2], h[3]);
+            if (GRADS) {
+                *reinterpret_cast<float4*>(pc + 2 * t) = make_float4(g[0], g[1], g[2], g[3]);
+                *reinterpret_cast<float4*>(pk + 2 * t) = make_float4(h[0], h[1], h[2], h[3]);
+            }
         } else {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 if (k0 + t + u < K) {
                     po[2 * (t + u)] = o[2 * u]; po[2 * (t + u) + 1] = o[2 * u + 1];
-                    pc[2 * (t + u)] = g[2 * u]; pc[2 * (t + u) + 1] = g[2 * u + 1];
-                    pk[2 * (t + u)] = h[2 * u]; pk[2 * (t + u) + 1] = h[2 * u + 1];
+                    if (GRADS) {
+                        pc[2 * (t + u)] = g[2 * u]; pc[2 * (t + u) + 1] = g[2 * u + 1];
+                        pk[2 * (t + u)] = h[2 * u]; pk[2 * (t + u) + 1] = h[2 * u + 1];
+                    }
                 }
             }
         }
@@ -321,14 +333,14 @@ const WaVariant kVariants[] = {
 };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
-template <int KT, bool SPLIT>
+template <int KT, bool SPLIT, bool GRADS>
 int launch(const float* ca, const float* cbv, int layout, const float* cbm, const float* wn, const uint8_t* mask,
            float* out, float* d_cb, float* d_k, int Z, int N, int K, hipStream_t st)
 {
     const int iblocks = (N + 63) / 64;
     const int ktiles  = SPLIT ? (K + KT - 1) / KT : (K + KT * WA_WAVES - 1) / (KT * WA_WAVES);
     dim3 grid(iblocks, ktiles, Z);
-    hipLaunchKernelGGL((we_aniso_fwd_kernel<KT, SPLIT>), grid, dim3(WA_THREADS), 0, st,
+    hipLaunchKernelGGL((we_aniso_fwd_kernel<KT, SPLIT, GRADS>), grid, dim3(WA_THREADS), 0, st,
                        ca, cbv, layout, cbm, wn, mask, out, d_cb, d_k, N, K);
     return (int)hipGetLastError();
 }
@@ -347,12 +359,13 @@ extern "C" int proteus_we_aniso_fwd_check(const float* coordsA, const float* coo
                                           int Z, int N, int K, int tuning)
 {
     (void)mask;
-    if (!coordsA || !coordsB || !cb_magnitudes || !wavenumbers || !out || !d_cb || !d_k) return PROTEUS_ERR_NULL_POINTER;
+    if (!coordsA || !coordsB || !cb_magnitudes || !wavenumbers || !out) return PROTEUS_ERR_NULL_POINTER;
+    if ((d_cb == nullptr) != (d_k == nullptr)) return PROTEUS_ERR_NULL_POINTER;       // both derivatives or neither
     if (Z <= 0 || N <= 0 || K <= 0) return PROTEUS_ERR_BAD_SHAPE;
     if (N > PROTEUS_WE_MAX_N || K > PROTEUS_WE_MAX_K || Z > 65535) return PROTEUS_ERR_BAD_SHAPE;
     if (coords_layout != PROTEUS_COORDS_SOA && coords_layout != PROTEUS_COORDS_AOS) return PROTEUS_ERR_BAD_LAYOUT;
     if (tuning < 0 || tuning >= kNumVariants) return PROTEUS_ERR_BAD_TUNING;
-    if (((uintptr_t)out & 15) || ((uintptr_t)d_cb & 15) || ((uintptr_t)d_k & 15)) return PROTEUS_ERR_BAD_ALIGNMENT;
+    if (((uintptr_t)out & 15) || ((uintptr_t)d_cb & 15) || ((uintptr_t)d_k & 15)) return PROTEUS_ERR_BAD_ALIGNMENT;   // (NULL passes)
     return PROTEUS_OK;
 }
 
@@ -369,27 +382,33 @@ extern "C" int proteus_we_aniso_fwd(const float* coordsA, const float* coordsB, 
     int kt = kVariants[tuning].kt;
     bool split = kVariants[tuning].split;
     if (tuning == 0) {
-        // Eight wavenumbers per wave measured faster than sixteen at every size tried (92 VGPRs, five
-        // waves per SIMD, against 157 and three), so only the source split is chosen here: by the least
-        // estimated issue time, instructions per wave x rounds of 1024 waves, with a penalty when a SIMD
-        // would hold a single wave.  A tie keeps the unsplit kernel.
-        kt = 8;
+        // With the partial derivatives (six sums per wavenumber) eight wavenumbers per wave measured faster than sixteen
+        // at every size tried (92 VGPRs, five waves per SIMD, against 155 and three); the embedding alone (two sums)
+        // is fastest with sixteen and the source split wherever the split is possible.  The split itself is chosen by
+        // the least estimated issue time, instructions per wave x rounds of 1024 waves, with a penalty when a SIMD
+        // would hold a single wave; a tie goes to the split kernel (measured 4 % faster at N = 16384 and at 8 x 1024).
+        kt = d_cb ? 8 : (N >= 4 * 64 ? 16 : 8);
         const long iblocks = ((long)N + 63) / 64 * Z;
         const long ktiles  = ((long)K + kt - 1) / kt;
         double best = 1e300;
-        for (int csp = 0; csp < 2; ++csp) {
+        for (int csp = 1; csp >= 0; --csp) {
             if (csp && N < 4 * 64) continue;
             const long nwaves = csp ? iblocks * ktiles * WA_WAVES : iblocks * ((ktiles + WA_WAVES - 1) / WA_WAVES) * WA_WAVES;
             const double keys = csp ? (double)N / WA_WAVES : (double)N;
             const double rounds = (double)((nwaves + 1023) / 1024);
-            double est = rounds * keys * (13.0 * kt + 22.0);
+            double est = rounds * keys * ((d_cb ? 13.0 : 9.0) * kt + 22.0);
             if (nwaves < 2048) est *= 1.25;
             if (est < best * 0.999) { best = est; split = csp != 0; }
         }
+        if (!d_cb && N >= 4 * 64) split = true;
     }
-#define WA_GO(KT_) (split ? launch<KT_, true>(coordsA, coordsB, coords_layout, cb_magnitudes, wavenumbers, mask, out, d_cb, d_k, Z, N, K, st) \
-                          : launch<KT_, false>(coordsA, coordsB, coords_layout, cb_magnitudes, wavenumbers, mask, out, d_cb, d_k, Z, N, K, st))
-    if (kt == 16) return WA_GO(16);
-    return WA_GO(8);
+#define WA_GO(KT_, GR_) (split ? launch<KT_, true, GR_>(coordsA, coordsB, coords_layout, cb_magnitudes, wavenumbers, mask, out, d_cb, d_k, Z, N, K, st) \
+                               : launch<KT_, false, GR_>(coordsA, coordsB, coords_layout, cb_magnitudes, wavenumbers, mask, out, d_cb, d_k, Z, N, K, st))
+    if (d_cb) {
+        if (kt == 16) return WA_GO(16, true);
+        return WA_GO(8, true);
+    }
+    if (kt == 16) return WA_GO(16, false);
+    return WA_GO(8, false);
 #undef WA_GO
 }

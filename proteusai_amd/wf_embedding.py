@@ -145,8 +145,11 @@ def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None
     return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask)
 
 
-def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tuning: int = 0):
+def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tuning: int = 0, partials: bool = True):
     """out, d_cb, d_k = we_aniso_forward(coordsA [Z,N,3], coordsB [Z,N,3], cb_magnitudes [K], wavenumbers [K], mask).
+
+    partials=False: only the embedding is computed (d_cb and d_k come back as None): the kernel keeps two running sums
+    per wavenumber instead of six.
 
     coordsA: token positions; coordsB: per-token C-beta direction vectors (relative to the token);
     mask [Z,N] bool, True = padded (None = nothing padded).  All outputs float32 [Z,N,2K], cos/real
@@ -177,15 +180,15 @@ def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tu
             raise ValueError(f"mask must be of shape ({Z}, {N}), not {tuple(mask.shape)}")
         m = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
     out = torch.empty(Z, N, 2 * K, dtype=torch.float32, device=dev)
-    d_cb = torch.empty_like(out)
-    d_k = torch.empty_like(out)
+    d_cb = torch.empty_like(out) if partials else None
+    d_k = torch.empty_like(out) if partials else None
     if Z == 0 or N == 0 or K == 0:
         return out, d_cb, d_k
     with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         rc = lib.proteus_we_aniso_fwd(a.data_ptr(), b.data_ptr(), _lib.COORDS_AOS, cb.data_ptr(), w.data_ptr(),
                                       None if m is None else m.data_ptr(),
-                                      out.data_ptr(), d_cb.data_ptr(), d_k.data_ptr(),
+                                      out.data_ptr(), d_cb.data_ptr() if partials else None, d_k.data_ptr() if partials else None,
                                       Z, N, K, int(tuning), stream)
     _lib.check(rc, "proteus_we_aniso_fwd")
     return out, d_cb, d_k
@@ -198,13 +201,18 @@ class _wf_embedding_learnCB(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask):
-        out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask)
-        ctx.save_for_backward(d_cb, d_k)
+        # the per-token partial derivatives are computed only if one of the two scales can want a gradient
+        ctx.need = bool(cb_magnitudes.requires_grad or wavenumbers.requires_grad)
+        out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask, partials=ctx.need)
+        if ctx.need:
+            ctx.save_for_backward(d_cb, d_k)
         ctx.dtypes = (cb_magnitudes.dtype, wavenumbers.dtype)
         return out.to(coordsA.dtype)
 
     @staticmethod
     def backward(ctx, dO):
+        if not ctx.need:
+            return None, None, None, None, None
         d_cb, d_k = ctx.saved_tensors
         g_cb, g_k = we_aniso_backward(dO, d_cb if ctx.needs_input_grad[2] else None,
                                       d_k if ctx.needs_input_grad[3] else None)

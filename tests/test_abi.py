@@ -70,6 +70,7 @@ def test_we_aniso_argument_validation():
     assert call() == 0
     for name in ("a", "b", "cb", "wn", "out", "dcb", "dk"):
         assert call(**{name: None}) == -1
+    assert call(dcb=None, dk=None) == 0               # only the embedding is wanted: both partials absent, not one
     for name in ("Z", "N", "K"):
         assert call(**{name: 0}) == -2
     assert call(N=(1 << 22) + 1) == -2 and call(K=4097) == -2

@@ -162,6 +162,28 @@ def test_autograd_function_and_module(gpu):
     assert rel_l2(y.detach().cpu().numpy(), r.numpy()) <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("tuning", range(0, 5))
+def test_embedding_alone_equals_the_embedding_with_partials(gpu, tuning):
+    # without the partial derivatives the kernel keeps two of the six running sums: the same additions in the same
+    # order, so with the variant fixed the embedding is the same to the bit (tuning 0 may pick another variant: 1e-6)
+    a, b, cb, wn, mask = inputs(333, seed=9, batch=2, K=40, pad=0.2)
+    full = run_gpu(gpu, a, b, cb, wn, mask, tuning=tuning)[0]
+    lean, d_cb, d_k = pa.we_aniso_forward(a.to(gpu), b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu), tuning=tuning, partials=False)
+    assert d_cb is None and d_k is None
+    lean = lean.cpu().numpy()
+    if tuning:
+        np.testing.assert_array_equal(lean, full)
+    else:
+        assert rel_l2(lean, full) <= 1e-6
+    # and the module takes that path when no scale is learnt
+    with torch.no_grad():
+        y = pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu)).cpu().numpy()
+    assert rel_l2(y, full) <= 1e-6
+    c = a.to(gpu).requires_grad_(True)                    # some other input wants a gradient: backward returns none for all
+    pa.wf_embedding_learnCB(c, b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu)).sum().backward()
+    assert c.grad is None
+
+
 def test_raw_c_abi_soa_layout_and_stream(gpu):
     a, b, cb, wn, mask = inputs(150, seed=9, batch=2, K=20, pad=0.15)
     lib = _lib.load()
