@@ -138,6 +138,60 @@ def test_forward_replays_bit_equal_from_a_captured_graph(gpu):
             assert torch.equal(out[~mask], eager[~mask])
 
 
+def test_operators_forward_and_backward_replay_from_a_captured_graph(gpu):
+    """The attention forward and backward and the embedding forward and backward, through their autograd functions,
+    captured into one graph: replays (with eager work between them) reproduce the eager gradients, to the bit except
+    d_sigma, which is summed with atomic adds.  (A whole training step is not captured here: some of torch's own
+    reductions record memset nodes, which this test does not mean to cover.)"""
+    g = torch.Generator().manual_seed(7)
+    Z, H, N, d = 2, 4, 700, 64
+    Q, K, V, coords, sigma, _ = synth.attn_inputs(Z, H, N, d, 7)
+    mask = torch.zeros(Z, N, dtype=torch.bool)
+    mask[1, 500:] = True
+    dO = (torch.randn(Z, H, N, d, generator=g) / 8).to(gpu)
+    dE = torch.randn(Z, N, 64, generator=g).to(gpu)
+    q, k, v = (t.to(gpu).requires_grad_(True) for t in (Q, K, V))
+    s = sigma.to(gpu).requires_grad_(True)
+    wn = torch.exp(torch.linspace(-1.0, 0.5, 32)).to(gpu).requires_grad_(True)
+    c, m = coords.to(gpu), mask.to(gpu)
+    leaves = (q, k, v, s, wn)
+
+    def step():
+        for t in leaves:
+            t.grad.zero_()
+        pa.geometric_attn(q, k, v, c, s, None, m, check_spreads=False).backward(dO)      # (the check reads sigma on the host)
+        pa.wf_embedding(c, wn, mask=m).backward(dE)
+
+    for t in leaves:
+        t.grad = torch.zeros_like(t)
+    step()
+    torch.cuda.synchronize()
+    eager = [t.grad.clone() for t in leaves]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        step()                                              # eager work between the replays
+        torch.cuda.synchronize()
+        for t in leaves:
+            t.grad.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for t, e, name in zip(leaves, eager, ("dQ", "dK", "dV", "d_sigma", "d_wavenumbers")):
+            if name == "d_sigma":
+                assert torch.allclose(t.grad, e, rtol=1e-5, atol=1e-9), name
+            else:
+                assert torch.equal(t.grad, e), name
+
+
 def test_training_step_through_both_kernels(gpu):
     # forward and backward of the whole stack on the HIP kernels (attention backward, wavenumber backward of the
     # embedding), one SGD step, and the loss goes down
