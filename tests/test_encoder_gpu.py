@@ -141,8 +141,8 @@ def test_forward_replays_bit_equal_from_a_captured_graph(gpu):
 def test_operators_forward_and_backward_replay_from_a_captured_graph(gpu):
     """The attention forward and backward and the embedding forward and backward, through their autograd functions,
     captured into one graph: replays (with eager work between them) reproduce the eager gradients, to the bit except
-    d_sigma, which is summed with atomic adds.  (A whole training step is not captured here: some of torch's own
-    reductions record memset nodes, which this test does not mean to cover.)"""
+    d_sigma, which is summed with atomic adds.  (A whole training step is not captured here: torch's own many-block
+    reductions, the bias gradients' column sums, clear their accumulators with memset nodes that replays do not repeat.)"""
     g = torch.Generator().manual_seed(7)
     Z, H, N, d = 2, 4, 700, 64
     Q, K, V, coords, sigma, _ = synth.attn_inputs(Z, H, N, d, 7)
