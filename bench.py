@@ -429,6 +429,13 @@ def main():
             "model_ms": slots * t_b * 1e3, "frac": slots * t_b * 1e3 / a_ms,
             "matrix_only_ms": slots * t_m * 1e3,
         }
+        # which vector instructions run beside a matrix product: the same loop with the softmax work replaced by
+        # twelve ordinary fused multiply-adds, and by four exp2 (ns per slot and SIMD: alone, and with the product)
+        t_pa, t_pm, t_ta, t_tm = (probe_slot_ms(lib, torch, dev, m) for m in (3, 4, 5, 6))
+        leg["roofline"]["issue_model"]["beside_a_product_ns"] = {
+            "twelve_fma": {"alone": t_pa * 1e9, "with_product": t_pm * 1e9, "hidden_frac": (t_m + t_pa - t_pm) / t_pa},
+            "four_exp2": {"alone": t_ta * 1e9, "with_product": t_tm * 1e9, "hidden_frac": (t_m + t_ta - t_tm) / t_ta},
+        }
         pa_ = read_profile(PROFILE_ATTN)
         if "mfma_util" in pa_:
             leg["roofline"]["mfma_util"] = {"value": pa_["mfma_util"], "mfma_flop_counted": pa_.get("mfma_flop"),

@@ -371,7 +371,10 @@ int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, in
  * Co-issue probe behind the attention forward's issue model (no counterpart in the reference).  Every wave runs
  * `iters` loop trips of eight "slots"; a slot is what the attention kernel's inner loop issues per 32x32x16 bf16
  * matrix product: that product and the softmax work of two scores (2 fused multiply-adds, 2 exp2, 1 pack to bf16,
- * 1 packed row-sum add).  mode 0: the matrix products only; 1: the vector work only; 2: both.  `blocks`
+ * 1 packed row-sum add).  mode 0: the matrix products only; 1: the vector work only; 2: both.  Modes 3-6 replace
+ * the vector work, to tell which kind of vector instruction runs beside a matrix product: 3: twelve ordinary fused
+ * multiply-adds per slot, alone; 4: those with the products; 5: four exp2 per slot, alone; 6: those with the
+ * products.  `blocks`
  * workgroups of 256 threads (512 on a 256-CU chip = two waves per SIMD, the attention kernel's occupancy);
  * sink [blocks*256] f32 receives values that keep the work alive.  Time the launch with events.
  */

@@ -89,7 +89,9 @@ typedef float  floatx2 __attribute__((ext_vector_type(2)));
 // One "slot" of the attention forward's inner loop: a 32x32x16 bf16 matrix product and the softmax work of two scores
 // (two fused multiply-adds, two exp2, one pack to bf16, one packed row-sum add).  MODE 0: the products only;
 // 1: the vector work only; 2: both, in the order the kernel issues them.  Eight slots per loop trip.
-template <int MODE>
+// VEC picks the vector work of a slot: 0 the softmax work; 1 twelve ordinary fused multiply-adds (about as long);
+// 2 four exp2 and nothing else.  The two last ones tell which kind of vector instruction runs beside a product.
+template <int MODE, int VEC>
 __global__ __launch_bounds__(256)
 void mfma_softmax_slot_kernel(float* sink, int iters) {
     floatx16 acc;
@@ -108,6 +110,19 @@ void mfma_softmax_slot_kernel(float* sink, int iters) {
             if (MODE != 1) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
             if (MODE != 0) {
                 asm volatile("" : "+v"(s0), "+v"(s1));          // opaque: nothing of the step is hoisted out of the loop
+                if (VEC == 1) {
+#pragma unroll
+                    for (int q = 0; q < 6; ++q) { s0 = __builtin_fmaf(s0, log2e, mneg); s1 = __builtin_fmaf(s1, log2e, mneg); }
+                    __builtin_amdgcn_sched_barrier(0);
+                    continue;
+                }
+                if (VEC == 2) {
+                    const float y0 = __builtin_amdgcn_exp2f(s0), y1 = __builtin_amdgcn_exp2f(s1);
+                    const float y2 = __builtin_amdgcn_exp2f(mneg), y3 = __builtin_amdgcn_exp2f(log2e);
+                    asm volatile("" :: "v"(y0), "v"(y1), "v"(y2), "v"(y3));
+                    __builtin_amdgcn_sched_barrier(0);
+                    continue;
+                }
                 const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0, log2e, mneg));
                 const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1, log2e, mneg));
                 const floatx2 f = {x0, x1};
@@ -117,7 +132,7 @@ void mfma_softmax_slot_kernel(float* sink, int iters) {
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    float s = lsum;
+    float s = lsum + s0 + s1;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s += acc[r];
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
@@ -128,11 +143,19 @@ void mfma_softmax_slot_kernel(float* sink, int iters) {
 extern "C" int proteus_probe_mfma_softmax_slot(int mode, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;
     if (blocks <= 0 || iters <= 0 || blocks > (1 << 20)) return PROTEUS_ERR_BAD_SHAPE;
-    if (mode < 0 || mode > 2) return PROTEUS_ERR_BAD_TUNING;
+    if (mode < 0 || mode > 6) return PROTEUS_ERR_BAD_TUNING;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (mode == 0)      hipLaunchKernelGGL((mfma_softmax_slot_kernel<0>), dim3(blocks), dim3(256), 0, st, sink, iters);
-    else if (mode == 1) hipLaunchKernelGGL((mfma_softmax_slot_kernel<1>), dim3(blocks), dim3(256), 0, st, sink, iters);
-    else                hipLaunchKernelGGL((mfma_softmax_slot_kernel<2>), dim3(blocks), dim3(256), 0, st, sink, iters);
+#define PROTEUS_SLOT(M_, V_) hipLaunchKernelGGL((mfma_softmax_slot_kernel<M_, V_>), dim3(blocks), dim3(256), 0, st, sink, iters)
+    switch (mode) {
+        case 0: PROTEUS_SLOT(0, 0); break;
+        case 1: PROTEUS_SLOT(1, 0); break;
+        case 2: PROTEUS_SLOT(2, 0); break;
+        case 3: PROTEUS_SLOT(1, 1); break;
+        case 4: PROTEUS_SLOT(2, 1); break;
+        case 5: PROTEUS_SLOT(1, 2); break;
+        default: PROTEUS_SLOT(2, 2); break;
+    }
+#undef PROTEUS_SLOT
     return (int)hipGetLastError();
 }
 

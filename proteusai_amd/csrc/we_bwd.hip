@@ -108,10 +108,10 @@ void we_bwd_partial_kernel(const float* __restrict__ d_out, const float* __restr
     }
 }
 
-// out_o[k] = sum over the slabs.  A workgroup takes WB_FK wavenumbers; WB_THREADS / WB_FK lanes share each
-// wavenumber's slabs (lane j takes slabs j, j + lanes, ...: independent loads, many in flight) and their partial
-// sums meet in LDS in a fixed order.
-constexpr int WB_FK = 16;
+// out_o[k] = sum over the slabs.  A workgroup takes WB_FK wavenumbers (few of them: many small workgroups are done
+// sooner than few large ones); WB_THREADS / WB_FK lanes share each wavenumber's slabs (lane j takes slabs j,
+// j + lanes, ...: independent loads, many in flight) and their partial sums meet in LDS in a fixed order.
+constexpr int WB_FK = 4;
 __global__ __launch_bounds__(WB_THREADS)
 void we_bwd_final_kernel(const float* __restrict__ partial, float* __restrict__ out0, float* __restrict__ out1,
                          const int slabs, const int K, const int n_out)
