@@ -588,6 +588,30 @@ def main():
         result["encoder_forward_backward"] = {"workload": "the same stack and batch, forward + backward (dropout 0)",
                                               "ms": e0.elapsed_time(e1) / 10}
 
+        # the layer's fused residual add + LayerNorm on its own: at the encoder's shape and at a size HBM can show
+        lnr = {}
+        for rows_ln, tag in ((8 * 1024, "encoder_shape"), (256 * 1024, "large")):
+            xa = torch.randn(rows_ln, 512, device=dev).bfloat16()
+            xb = torch.randn(rows_ln, 512, device=dev).bfloat16()
+            ga, be = torch.ones(512, device=dev).bfloat16(), torch.zeros(512, device=dev).bfloat16()
+            xo = torch.empty_like(xa)
+
+            def ln_step():
+                rc = lib.proteus_add_layernorm_fwd(xa.data_ptr(), xb.data_ptr(), ga.data_ptr(), be.data_ptr(), xo.data_ptr(),
+                                                   rows_ln, 512, 1e-5, _lib.DTYPE_BF16, stream)
+                if rc != 0:
+                    _lib.check(rc, "proteus_add_layernorm_fwd")
+            _, ln_ms = time_launches(torch, ln_step, 20)
+            ln_bytes = 3.0 * 2 * rows_ln * 512                 # x, res in; out: bf16
+            lnr[tag] = {"rows": rows_ln, "ms": ln_ms, "GB_per_s": ln_bytes / (ln_ms * 1e-3) / 1e9}
+            del xa, xb, xo
+        result["add_layernorm"] = {
+            "workload": "residual add + LayerNorm over 512 features, bf16 (the encoder layer's two normalisations; inference path)",
+            "dtype": "bf16", **lnr,
+            "roofline": {"kernel": "add_layernorm_kernel", "bound": "hbm", "achieved": lnr["large"]["GB_per_s"], "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": lnr["large"]["GB_per_s"] / PEAK_HBM_GBS, "traffic": None},
+        }
+
     # ---------------- CPU baseline of the headline shape: the tiled CPU PyTorch path on a bounded sample of observer rows --------
     if not args.no_cpu:
         if args.full_cpu:

@@ -38,11 +38,15 @@ extern "C" {
 #define PROTEUS_ERR_BAD_TUNING    -6   /* unknown tuning/variant selector         */
 #define PROTEUS_ERR_UNSUPPORTED   -7   /* legacy option not implemented           */
 #define PROTEUS_ERR_TOO_LARGE     -8   /* beyond the fixed capacity of an entry point that allocates nothing */
-#define PROTEUS_ERR_BAD_OPERAND_TYPE -9 /* operand_type is neither PROTEUS_OPERAND_BF16 nor PROTEUS_OPERAND_F16 */
+#define PROTEUS_ERR_BAD_OPERAND_TYPE -9 /* operand_type is neither PROTEUS_OPERAND_BF16 nor PROTEUS_OPERAND_F16 (dtype: neither PROTEUS_DTYPE_*) */
 
 /* 16-bit type of Q, K, V (and dO) where an entry point takes an operand_type */
 #define PROTEUS_OPERAND_BF16 0
 #define PROTEUS_OPERAND_F16  1
+
+/* element type of the tensors of proteus_add_layernorm_fwd */
+#define PROTEUS_DTYPE_F32  0
+#define PROTEUS_DTYPE_BF16 1
 
 /* ---- coordinate layouts accepted by proteus_we_fwd ---- */
 #define PROTEUS_COORDS_SOA 0   /* [Z,3,N]: what the reference's wrapper hands its kernel */
@@ -345,6 +349,24 @@ int proteus_geo_attn_bwd_strided_check(const uint16_t* Q, const uint16_t* K, con
 
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);
+
+/*
+ * Residual add + LayerNorm of the post-LN encoder layer, inference forward:
+ *   out[r, :] = LayerNorm(x[r, :] + res[r, :]) * gamma + beta        over the last dimension D
+ * Replaces the torch expressions `self.attn_norm(q + self.dropout(attn))` and `self.ffn_norm(q + self.dropout(ffn))`
+ * of old/old_scripts/encoder.py:36-39 with dropout inactive (nn.LayerNorm(d_model), old/old_scripts/encoder.py:27,31),
+ * evaluated as torch does: the sum rounded to the tensors' type, mean and biased variance in fp32, eps under the
+ * square root.  One launch, HBM-bound, no workspace.
+ *   x, out        [rows, D] contiguous, dtype PROTEUS_DTYPE_F32 or PROTEUS_DTYPE_BF16 (all tensors of one type)
+ *   res           [rows, D] or NULL (plain LayerNorm)
+ *   gamma, beta   [D] or NULL (no scale / no shift)
+ *   D             a multiple of 4 (f32) or 8 (bf16), at most 2048 (f32) or 4096 (bf16); pointers 16-byte aligned
+ *   out may be x or res (every row is read completely before it is written)
+ */
+int proteus_add_layernorm_fwd(const void* x, const void* res, const void* gamma, const void* beta, void* out,
+                              long rows, int D, float eps, int dtype, void* stream);
+int proteus_add_layernorm_fwd_check(const void* x, const void* res, const void* gamma, const void* beta, const void* out,
+                                    long rows, int D, float eps, int dtype);
 
 /*
  * Instruction-rate probe used to state the roofline denominator of the WE

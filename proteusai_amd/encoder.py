@@ -7,14 +7,46 @@ Follows the legacy transformer architecture the reference's README describes
   GeoAttention                 old/old_scripts/encoder.py:43-121  (proteusai_amd.geometric_attn.GeoAttention)
 The wavefunction embedding is added to an amino-acid embedding table and the
 sum runs through the encoder layers and a linear head to 20 amino-acid logits.
-Only plain PyTorch glue lives here; the two O(N^2) operators are the HIP kernels.
+Plain PyTorch glue but for the residual add + LayerNorm of a layer; the two O(N^2) operators are the HIP kernels.
 """
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import _lib
 from .geometric_attn import GeoAttention
 from .wf_embedding import WaveFunctionEmbedding
+
+
+def add_layer_norm(x, res, norm: nn.LayerNorm):
+    """norm(x + res) for the post-LN layer (old/old_scripts/encoder.py:36-39).
+
+    Where nothing needs a gradient (inference) and the tensors are fp32 or bf16 on the GPU, one HIP kernel reads x and
+    res once and writes the result (proteus_add_layernorm_fwd); otherwise the torch expression, which autograd
+    differentiates.  Both evaluate the same thing: the sum in the tensors' type, the statistics in fp32.
+    """
+    w, b = norm.weight, norm.bias
+    D = x.shape[-1]
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, res, w, b))
+    fused = (not needs_grad and x.is_cuda and x.dtype in (torch.float32, torch.bfloat16) and res.dtype == x.dtype
+             and x.shape == res.shape and tuple(norm.normalized_shape) == (D,)
+             and all(t is None or t.dtype == x.dtype for t in (w, b))
+             and D % (4 if x.dtype == torch.float32 else 8) == 0 and D <= (2048 if x.dtype == torch.float32 else 4096))
+    if not fused:
+        return norm(x + res)
+    lib = _lib.load()
+    xc, rc_ = x.contiguous(), res.contiguous()
+    out = torch.empty_like(xc)
+    rows = xc.numel() // D
+    if rows == 0:
+        return out
+    with _lib.on_device(x.device):
+        rc = lib.proteus_add_layernorm_fwd(xc.data_ptr(), rc_.data_ptr(), None if w is None else w.data_ptr(),
+                                           None if b is None else b.data_ptr(), out.data_ptr(), rows, D, float(norm.eps),
+                                           _lib.DTYPE_F32 if x.dtype == torch.float32 else _lib.DTYPE_BF16,
+                                           torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "proteus_add_layernorm_fwd")
+    return out
 
 
 class MLP(nn.Module):
@@ -56,8 +88,8 @@ class Encoder(nn.Module):
         self.dropout = nn.Dropout(dropout)
 
     def forward(self, q, k, v, coords, mask=None):
-        q = self.attn_norm(q + self.dropout(self.attn(q, k, v, coords, mask=mask)))
-        q = self.ffn_norm(q + self.dropout(self.ffn(q)))
+        q = add_layer_norm(q, self.dropout(self.attn(q, k, v, coords, mask=mask)), self.attn_norm)
+        q = add_layer_norm(q, self.dropout(self.ffn(q)), self.ffn_norm)
         return q
 
 

@@ -303,8 +303,19 @@ class GeoAttention(nn.Module):
         # projection.  Token-major O is the (heads x d_k) order; the same product is taken against the projection's
         # input columns in that order instead of reshuffling the activations.
         out = out.permute(0, 2, 1, 3).reshape(batch, N, self.d_model)           # a view when O is token-major
-        w_o = self.out_proj.weight.view(self.d_model, dk, H).permute(0, 2, 1).reshape(self.d_model, self.d_model)
-        return torch.nn.functional.linear(out, w_o)
+        return torch.nn.functional.linear(out, self._out_weight())
+
+    def _out_weight(self):
+        """The output projection's weight with its input columns in (heads x d_k) order.  Rebuilt whenever the
+        parameter may have changed; kept across calls only where no gradient is needed."""
+        p = self.out_proj.weight
+        keep = not (torch.is_grad_enabled() and p.requires_grad)
+        key = (p._version, p.data_ptr(), p.dtype)
+        if keep and getattr(self, "_wo_cache", None) is not None and self._wo_cache[0] == key:
+            return self._wo_cache[1]
+        w_o = p.view(self.d_model, self.d_k, self.heads).permute(0, 2, 1).reshape(self.d_model, self.d_model)
+        self._wo_cache = (key, w_o.detach()) if keep else None
+        return w_o
 
     def _fused_qkv(self):
         """[d_model, 3*H*d_k] weight and [3*H*d_k] bias of the fused self-attention projection.  Rebuilt from the

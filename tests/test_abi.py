@@ -303,3 +303,24 @@ def test_strided_attention_argument_validation():
     assert bwd(None) == -1
     assert bwd(arr(*(plain * 6 + [H * N * 64, N * 64, 63]))) == -4
     assert bwd(arr(*(plain * 6 + [H * N * 64, N * 64, 66]))) == -5
+
+
+def test_add_layernorm_argument_validation():
+    lib = _lib.load()
+    p = 0x1000
+    f32, bf16 = _lib.DTYPE_F32, _lib.DTYPE_BF16
+
+    def chk(x=p, res=p, gamma=p, beta=p, out=p, rows=10, D=512, eps=1e-5, dtype=bf16):
+        return lib.proteus_add_layernorm_fwd_check(x, res, gamma, beta, out, rows, D, eps, dtype)
+    assert chk() == 0 and chk(dtype=f32) == 0
+    assert chk(res=None, gamma=None, beta=None) == 0                 # plain normalisation
+    assert chk(out=p, x=p) == 0                                      # in place
+    assert chk(x=None) == -1 and chk(out=None) == -1
+    assert chk(dtype=2) == -9
+    assert chk(rows=0) == -2 and chk(D=0) == -2
+    assert chk(D=4096) == 0 and chk(D=4104) == -2                    # bf16: at most 4096
+    assert chk(D=2048, dtype=f32) == 0 and chk(D=2052, dtype=f32) == -2
+    assert chk(D=516) == -2 and chk(D=516, dtype=f32) == 0           # multiples of 8 (bf16), 4 (fp32)
+    assert chk(eps=-1.0) == -2 and chk(eps=float("nan")) == -2
+    assert chk(x=p + 8) == -5 and chk(gamma=p + 4) == -5
+    assert lib.proteus_add_layernorm_fwd(None, p, p, p, p, 10, 512, 1e-5, bf16, None) == -1
