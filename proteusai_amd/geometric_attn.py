@@ -293,17 +293,30 @@ class GeoAttention(nn.Module):
             V = heads_first(torch.addmm(self.v_bias.reshape(-1), v.reshape(batch * N, d_model), flat(self.v_proj)))
         # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
         if self.legacy_logits:
-            out = geometric_attn(Q, K, V, coords, self.get_spreads(), self.get_betas(), mask=mask, min_rbf=self.min_rbf,
+            out = geometric_attn(Q, K, V, coords, self._per_head("spread"), self._per_head("beta"), mask=mask, min_rbf=self.min_rbf,
                                  max_rbf=self.max_rbf, check_spreads=False, token_major_out=True, out_dtype=q.dtype,
                                  operand_dtype=self.operand_dtype)
         else:
-            out = geometric_attn(Q, K, V, coords, self.get_spreads(), None, mask=mask, check_spreads=False,
+            out = geometric_attn(Q, K, V, coords, self._per_head("spread"), None, mask=mask, check_spreads=False,
                                  token_major_out=True, out_dtype=q.dtype)
         # The reference concatenates the heads as a (d_k x heads) interleave (encoder.py:114-115) before the output
         # projection.  Token-major O is the (heads x d_k) order; the same product is taken against the projection's
         # input columns in that order instead of reshuffling the activations.
         out = out.permute(0, 2, 1, 3).reshape(batch, N, self.d_model)           # a view when O is token-major
         return torch.nn.functional.linear(out, self._out_weight())
+
+    def _per_head(self, which):
+        """sigma (`spread`) or beta of the heads.  Where no gradient is needed the fp32 values the kernel reads are
+        kept across calls (three small launches per layer otherwise) until the parameter changes."""
+        p = self.spread_weights if which == "spread" else self.beta_weights
+        fn = self.get_spreads if which == "spread" else self.get_betas
+        if torch.is_grad_enabled() and p.requires_grad:
+            return fn()
+        key = (p._version, p.data_ptr(), p.dtype, self.min_spread)
+        cache = self.__dict__.setdefault("_head_cache", {})
+        if which not in cache or cache[which][0] != key:
+            cache[which] = (key, fn().detach().float().contiguous())
+        return cache[which][1]
 
     def _out_weight(self):
         """The output projection's weight with its input columns in (heads x d_k) order.  Rebuilt whenever the
