@@ -68,7 +68,11 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     const uint8_t* mz = mask ? mask + zN : nullptr;
 
     // ---- this lane's observer ----
-    const int  i    = blockIdx.x * 64 + lane;
+    // (observer blocks taken in a rotated order per (y, z), as in the isotropic kernel: in a batch of ragged lengths the
+    // workgroups that are resident together then belong to different parts of their sequences)
+    const unsigned wa_rot = ((unsigned)(0.6180339887f * (float)gridDim.x + 0.5f)) | 1u;
+    const int  iblock = (int)((blockIdx.x + wa_rot * (blockIdx.z % gridDim.x) + 5u * blockIdx.y) % gridDim.x);
+    const int  i    = iblock * 64 + lane;
     const bool i_in = i < N;
     const int  ic   = i_in ? i : N - 1;
     float xi, yi, zi;
