@@ -59,6 +59,42 @@ def test_cfg4_shape_bf16_and_padding_independence(gpu):
     assert torch.equal(out[valid], out2[valid])
 
 
+def test_cfg4_shape_inference_path_equals_the_path_autograd_records(gpu):
+    # Without gradients the layer's residual add + LayerNorm is one HIP kernel and the per-head constants are cached;
+    # with gradients enabled the torch expressions run.  Same weights, same batch: the two forwards differ only by
+    # how a bf16 result was rounded here and there (fp32 weights: by fp32 rounding, which the attention's cast of its
+    # operands to bf16 turns into a flipped bf16 rounding now and then: measured 2.3e-4).
+    g = torch.Generator().manual_seed(4)
+    coords = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)]).to(gpu)
+    tokens = torch.randint(0, 33, (8, 1024), generator=g).to(gpu)
+    lens = torch.randint(128, 1025, (8,), generator=g)
+    mask = (torch.arange(1024)[None, :] >= lens[:, None]).to(gpu)
+    valid = ~mask.cpu()
+    for dtype, bar in ((torch.float32, 2e-3), (torch.bfloat16, 3e-2)):
+        torch.manual_seed(4)
+        model = pa.ProteusEncoder().eval().to(gpu)
+        model.aa_embedding.to(dtype)
+        model.layers.to(dtype)
+        model.head.to(dtype)
+        with torch.no_grad():
+            fast = model(coords, tokens, mask).float().cpu()
+        recorded = model(coords, tokens, mask)                      # parameters require gradients: the torch expressions
+        assert recorded.requires_grad
+        recorded = recorded.detach().float().cpu()
+        err = float((fast[valid] - recorded[valid]).norm() / recorded[valid].norm())
+        assert err <= bar, f"{dtype}: rel-L2 {err:.3e}"
+        # a second call reuses the cached constants: bit-equal
+        with torch.no_grad():
+            again = model(coords, tokens, mask).float().cpu()
+        assert torch.equal(fast[valid], again[valid])
+        # and they follow the parameter: a changed spread must change the result
+        with torch.no_grad():
+            for layer in model.layers:
+                layer.attn.spread_weights.add_(0.5)
+            moved = model(coords, tokens, mask).float().cpu()
+        assert not torch.equal(fast[valid], moved[valid])
+
+
 def test_cfg4_shape_embedding_and_first_attention_on_sampled_rows(gpu):
     """At the real shape (B=8, N=1024, d_model=512, H=8, bf16 weights, fp32 WE, lengths in [128, 1024]) a dense oracle of
     the whole stack takes too long for a test, but rows are independent in both kernels: the embedding and the first
