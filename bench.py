@@ -476,6 +476,19 @@ def main():
                              "unit": "TFLOP/s", "frac": 10.0 * 8 * 64 * 16384 * 16384 / (b_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
                              "traffic": b_traffic, "traffic_source": b_traffic_src},
             }
+            # D = rowsum(O * dO), taken before the backward kernel (its `D` argument): one pass over O (fp32) and dO (bf16)
+            Dk = torch.empty(1, 8, 16384, device=dev)
+
+            def delta_step():
+                rc = lib.proteus_geo_attn_delta(O.data_ptr(), dOb.data_ptr(), None, Dk.data_ptr(), 1, 8, 16384, 64, _lib.DTYPE_BF16, stream)
+                if rc != 0:
+                    _lib.check(rc, "proteus_geo_attn_delta")
+            _, d_ms = time_launches(torch, delta_step, 20)
+            d_bytes = 8.0 * 16384 * (64 * 6 + 4)
+            result["geo_attn_bwd"]["delta"] = {"kernel": "geo_attn_delta_kernel", "ms": d_ms, "bound": "hbm",
+                                               "achieved": d_bytes / (d_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                               "frac": d_bytes / (d_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                               "equals_torch": bool(torch.allclose(Dk, Dv, rtol=1e-5, atol=1e-6))}
             # ---- the reference kernel's own logits (beta-weighted bias, pair mask) at its module's default rbf range:
             #      key tiles whose pairs are all below min_rbf are skipped ----
             bet = torch.full((8,), 0.5, device=dev)

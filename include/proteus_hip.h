@@ -44,9 +44,10 @@ extern "C" {
 #define PROTEUS_OPERAND_BF16 0
 #define PROTEUS_OPERAND_F16  1
 
-/* element type of the tensors of proteus_add_layernorm_fwd */
+/* element type of the tensors of proteus_add_layernorm_fwd and of dO in proteus_geo_attn_delta */
 #define PROTEUS_DTYPE_F32  0
 #define PROTEUS_DTYPE_BF16 1
+#define PROTEUS_DTYPE_F16  2   /* proteus_geo_attn_delta only */
 
 /* ---- coordinate layouts accepted by proteus_we_fwd ---- */
 #define PROTEUS_COORDS_SOA 0   /* [Z,3,N]: what the reference's wrapper hands its kernel */
@@ -346,6 +347,22 @@ int proteus_geo_attn_bwd_strided_check(const uint16_t* Q, const uint16_t* K, con
                                        const float* dQ, const float* dK, const float* dV,
                                        const float* d_sigma, const float* d_beta,
                                        int Z, int H, int N, int d_head, float min_rbf, float max_rbf, int operand_type);
+
+/*
+ * D = rowsum(O * dO), the term the attention backward subtracts from dP.  Replaces the torch expression
+ * `D = torch.sum(O*dO, dim=3)` of the reference's backward wrapper (old/old_scripts/attn/geometric_attn.py:618);
+ * its result is the `D` argument of proteus_geo_attn_bwd.  One launch, HBM-bound, no workspace.
+ *   O        f32, rows of d_head elements contiguous and 16-byte aligned
+ *   dO       dO_dtype = PROTEUS_DTYPE_F32, _BF16 or _F16 (what autograd hands over, before any cast); rows of d_head
+ *            elements contiguous, starting on multiples of 4 elements
+ *   strides  NULL: both tensors contiguous [Z,H,N,d_head]; else 6 element strides, (batch, head, token) of O then of
+ *            dO, each a multiple of 4 and non-negative, token strides >= d_head
+ *   D        f32 [Z,H,N] contiguous
+ */
+int proteus_geo_attn_delta(const float* O, const void* dO, const int64_t* strides, float* D,
+                           int Z, int H, int N, int d_head, int dO_dtype, void* stream);
+int proteus_geo_attn_delta_check(const float* O, const void* dO, const int64_t* strides, const float* D,
+                                 int Z, int H, int N, int d_head, int dO_dtype);
 
 int         proteus_geo_attn_num_variants(void);
 const char* proteus_geo_attn_variant_name(int tuning);

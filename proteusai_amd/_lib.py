@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "libproteus_hip.so")
 COORDS_SOA = 0
 COORDS_AOS = 1
 OPERAND_BF16, OPERAND_F16 = 0, 1     # PROTEUS_OPERAND_* of include/proteus_hip.h
-DTYPE_F32, DTYPE_BF16 = 0, 1         # PROTEUS_DTYPE_*
+DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2   # PROTEUS_DTYPE_*
 
 # every symbol include/proteus_hip.h declares
 SYMBOLS = [
@@ -25,7 +25,7 @@ SYMBOLS = [
     "proteus_geo_attn_legacy_fwd_strided",
     "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
-    "proteus_add_layernorm_fwd", "proteus_add_layernorm_fwd_check",
+    "proteus_add_layernorm_fwd", "proteus_add_layernorm_fwd_check", "proteus_geo_attn_delta", "proteus_geo_attn_delta_check",
     "proteus_probe_valu_rate", "proteus_probe_sincos", "proteus_probe_mfma_softmax_slot",
 ]
 
@@ -110,6 +110,10 @@ def load():
     lib.proteus_add_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, ctypes.c_long, ci, cf, ci, vp]
     lib.proteus_add_layernorm_fwd_check.restype = ci
     lib.proteus_add_layernorm_fwd_check.argtypes = [vp, vp, vp, vp, vp, ctypes.c_long, ci, cf, ci]
+    lib.proteus_geo_attn_delta.restype = ci
+    lib.proteus_geo_attn_delta.argtypes = [vp, vp, i64p, vp, ci, ci, ci, ci, ci, vp]
+    lib.proteus_geo_attn_delta_check.restype = ci
+    lib.proteus_geo_attn_delta_check.argtypes = [vp, vp, i64p, vp, ci, ci, ci, ci, ci]
     lib.proteus_probe_valu_rate.restype = ci
     lib.proteus_probe_valu_rate.argtypes = [ci, ci, ci, vp, vp]
     lib.proteus_probe_sincos.restype = ci

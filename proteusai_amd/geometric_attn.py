@@ -130,6 +130,29 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     return (O, L) if return_lse else O
 
 
+_DELTA_DTYPES = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}
+
+
+def _delta(O, dO):
+    """D = rowsum(O * dO) [Z,H,N] fp32 (old/old_scripts/attn/geometric_attn.py:618), in one pass over both tensors
+    where their layout allows (rows of d contiguous, strides multiples of 4 elements); the torch expression otherwise."""
+    Z, H, N, d = O.shape
+    plain = (O.is_cuda and O.dtype == torch.float32 and dO.dtype in _DELTA_DTYPES and dO.shape == O.shape and d in (32, 64, 128)
+             and Z * H * N > 0 and Z * H <= 65535
+             and O.stride(3) == 1 and dO.stride(3) == 1 and O.stride(2) >= d and dO.stride(2) >= d
+             and all(s % 4 == 0 for s in O.stride()[:3] + dO.stride()[:3])
+             and O.data_ptr() % 16 == 0 and dO.data_ptr() % (4 * dO.element_size()) == 0)
+    if not plain:
+        return torch.sum(O.float() * dO, dim=3).contiguous()       # fp32 by type promotion
+    D = torch.empty(Z, H, N, dtype=torch.float32, device=O.device)
+    strides = None if (O.is_contiguous() and dO.is_contiguous()) else _lib.stride_array(O, dO)
+    with _lib.on_device(O.device):
+        rc = _lib.load().proteus_geo_attn_delta(O.data_ptr(), dO.data_ptr(), strides, D.data_ptr(), Z, H, N, d,
+                                                _DELTA_DTYPES[dO.dtype], torch.cuda.current_stream(O.device).cuda_stream)
+    _lib.check(rc, "proteus_geo_attn_delta")
+    return D
+
+
 def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, betas=None,
                       min_rbf: float = 0.0, max_rbf: float = 1.0, operand_dtype=None):
     """dQ, dK, dV [Z,H,N,d] f32, d_sigma [H] f32, d_betas [H] f32 | None from the forward's O and logsumexp L.
@@ -145,7 +168,7 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     dev = Q.device
     op_dtype, op_type = _operand_type(operand_dtype, betas is not None)
     q, k, v = _operand(Q, op_dtype), _operand(K, op_dtype), _operand(V, op_dtype)
-    D = torch.sum(O.detach().float() * dO.detach(), dim=3).contiguous()       # fp32 by type promotion
+    D = _delta(O.detach(), dO.detach())
     do = _operand(dO, op_dtype)
     c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
     s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()

@@ -324,3 +324,27 @@ def test_add_layernorm_argument_validation():
     assert chk(eps=-1.0) == -2 and chk(eps=float("nan")) == -2
     assert chk(x=p + 8) == -5 and chk(gamma=p + 4) == -5
     assert lib.proteus_add_layernorm_fwd(None, p, p, p, p, 10, 512, 1e-5, bf16, None) == -1
+
+
+def test_attention_delta_argument_validation():
+    import ctypes
+    lib = _lib.load()
+    p = 0x1000
+
+    def arr(*v):
+        return (ctypes.c_int64 * len(v))(*v)
+
+    def chk(O=p, dO=p, strides=None, D=p, Z=2, H=4, N=100, d=64, dtype=_lib.DTYPE_BF16):
+        return lib.proteus_geo_attn_delta_check(O, dO, strides, D, Z, H, N, d, dtype)
+    assert chk() == 0 and chk(dtype=_lib.DTYPE_F32) == 0 and chk(dtype=_lib.DTYPE_F16) == 0
+    assert chk(O=None) == -1 and chk(dO=None) == -1 and chk(D=None) == -1
+    assert chk(d=48) == -3 and chk(dtype=3) == -9
+    assert chk(N=0) == -2 and chk(Z=70000, H=1) == -2
+    assert chk(O=p + 8) == -5 and chk(dO=p + 4) == -5 and chk(dO=p + 8) == 0 and chk(dO=p + 8, dtype=_lib.DTYPE_F32) == -5
+    plain = [4 * 100 * 64, 100 * 64, 64]
+    tok = [100 * 4 * 64, 64, 4 * 64]
+    assert chk(strides=arr(*(plain + tok))) == 0
+    assert chk(strides=arr(*(plain + [4 * 100 * 64, 100 * 64, 32]))) == -4          # rows would overlap
+    assert chk(strides=arr(*([-4, 100 * 64, 64] + plain))) == -4
+    assert chk(strides=arr(*(plain + [4 * 100 * 64, 100 * 64, 66]))) == -5          # rows off the 4-element grid
+    assert lib.proteus_geo_attn_delta(None, p, None, p, 2, 4, 100, 64, _lib.DTYPE_BF16, None) == -1

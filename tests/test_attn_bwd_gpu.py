@@ -326,3 +326,39 @@ def test_strided_operands_give_the_same_gradients(gpu):
     Qh = dev(Q).permute(1, 0, 2, 3).contiguous().permute(1, 0, 2, 3)
     got2 = pa.geo_attn_backward(Qh, dev(K), dev(V), O, L, dev(dO).bfloat16(), dev(coords), dev(sigma), dev(mask))
     assert got2[0].stride() == Qh.stride() and torch.equal(got2[0], ref[0])
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_delta_rowsum_equals_the_torch_expression(gpu, d, dtype):
+    """D = rowsum(O * dO) (old/old_scripts/attn/geometric_attn.py:618) from proteus_geo_attn_delta: contiguous tensors,
+    token-major O with a differently laid out dO, and a slice of a wider buffer, against the fp64 sum of the same
+    products (fp32 products and sums: rel-L2 <= 1e-6, every row within 1e-5 of its sum of absolute products)."""
+    from proteusai_amd.geometric_attn import _delta
+    Z, H, N = 2, 3, 777
+    g = torch.Generator().manual_seed(d)
+    O = torch.randn(Z, H, N, d, generator=g)
+    dO = torch.randn(Z, H, N, d, generator=g).to(dtype)
+    ref = (O.double() * dO.double()).sum(-1)
+    scale = (O.double() * dO.double()).abs().sum(-1)
+
+    def check(D, what):
+        D = D.double().cpu()
+        assert D.shape == (Z, H, N) and torch.isfinite(D).all(), what
+        assert float((D - ref).norm() / ref.norm()) <= 1e-6, what
+        assert bool(((D - ref).abs() <= 1e-5 * scale).all()), what
+    check(_delta(O.to(gpu), dO.to(gpu)), "contiguous")
+    # O token-major ([Z,N,H,d] in memory), dO contiguous
+    Ot = O.permute(0, 2, 1, 3).contiguous().to(gpu).permute(0, 2, 1, 3)
+    assert not Ot.is_contiguous()
+    check(_delta(Ot, dO.to(gpu)), "token-major O")
+    # both as slices of buffers with room behind every row
+    wide_o = torch.zeros(Z, H, N, d + 8)
+    wide_o[..., :d] = O
+    wide_g = torch.zeros(Z, H, N, 2 * d, dtype=dtype)
+    wide_g[..., :d] = dO
+    check(_delta(wide_o.to(gpu)[..., :d], wide_g.to(gpu)[..., :d]), "sliced rows")
+    # a layout the kernel does not take (rows off the 16-byte grid) falls back to the torch expression
+    odd = torch.zeros(Z, H, N, d + 1)
+    odd[..., 1:] = O
+    check(_delta(odd.to(gpu)[..., 1:], dO.to(gpu)), "unaligned rows")
