@@ -154,12 +154,14 @@ def _delta(O, dO):
 
 
 def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, betas=None,
-                      min_rbf: float = 0.0, max_rbf: float = 1.0, operand_dtype=None):
+                      min_rbf: float = 0.0, max_rbf: float = 1.0, operand_dtype=None, grads=None):
     """dQ, dK, dV [Z,H,N,d] f32, d_sigma [H] f32, d_betas [H] f32 | None from the forward's O and logsumexp L.
 
     What the reference's wrapper does around its backward kernel (geometric_attn.py:609-660):
     D = rowsum(O*dO), dO cast to the operand type (bf16, or fp16 with operand_dtype=torch.float16 and betas), zeroed
     accumulators for the per-head scalars.
+    grads: optional (dQ, dK, dV) fp32 [Z,H,N,d] tensors to write into (rows of d contiguous, e.g. views of one
+    [Z,N,3,H,d] buffer); allocated here otherwise.
     """
     Z, H, N, d = Q.shape
     if not Q.is_cuda:
@@ -181,7 +183,13 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     def like(t):
         g = torch.empty_like(t, dtype=torch.float32)
         return g if _rows_ok(g, 4) else torch.empty(Z, H, N, d, dtype=torch.float32, device=dev)
-    dQ, dK, dV = like(Q), like(K), like(V)
+    if grads is None:
+        dQ, dK, dV = like(Q), like(K), like(V)
+    else:
+        dQ, dK, dV = grads
+        for g_ in grads:
+            if g_.dtype != torch.float32 or tuple(g_.shape) != (Z, H, N, d) or not _rows_ok(g_, 4):
+                raise AssertionError("grads must be fp32 [Z,H,N,d] tensors with contiguous, 16-byte aligned rows")
     d_sigma = torch.zeros(H, dtype=torch.float32, device=dev)
     d_beta = None if bt is None else torch.zeros(H, dtype=torch.float32, device=dev)
     if Z == 0 or H == 0 or N == 0:
@@ -223,6 +231,47 @@ class _geometric_attn(torch.autograd.Function):
                                                         ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype)
         return (dQ.to(Q.dtype), dK.to(K.dtype), dV.to(V.dtype), None, d_sigma.to(spreads.dtype),
                 None if betas is None else d_beta.to(betas.dtype), None, None, None, None, None, None, None)
+
+
+class _geometric_attn_qkv(torch.autograd.Function):
+    """The same operator on a fused projection qkv [Z,N,3,H,d] (self-attention: what one GEMM over the three
+    projections leaves).  Forward and backward read Q, K, V in place; the backward writes dQ, dK, dV into one
+    [Z,N,3,H,d] buffer, which is the gradient of qkv: no per-slice gradients for autograd to pad and add up."""
+
+    @staticmethod
+    def forward(ctx, qkv, coords, spreads, betas, key_padding_mask, min_rbf, max_rbf, check_sigma, out_dtype, operand_dtype):
+        Q, K, V = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        O, L = geo_attn(Q, K, V, coords, spreads, key_padding_mask, return_lse=True, betas=betas,
+                        min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_sigma, token_major_out=True,
+                        operand_dtype=operand_dtype)
+        ctx.save_for_backward(qkv, O, L, coords, spreads, betas, key_padding_mask)
+        ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype = min_rbf, max_rbf, operand_dtype
+        return O if out_dtype is None or out_dtype == O.dtype else O.to(out_dtype)
+
+    @staticmethod
+    def backward(ctx, dO):
+        qkv, O, L, coords, spreads, betas, mask = ctx.saved_tensors
+        Q, K, V = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        g = torch.empty(qkv.shape, dtype=torch.float32, device=qkv.device)
+        grads = tuple(g[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        _, _, _, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
+                                                     ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype, grads=grads)
+        return (g.to(qkv.dtype), None, d_sigma.to(spreads.dtype), None if betas is None else d_beta.to(betas.dtype),
+                None, None, None, None, None, None)
+
+
+def geometric_attn_qkv(qkv, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True,
+                       out_dtype=None, operand_dtype=None):
+    """geometric_attn for self-attention on a fused projection: qkv [Z,N,3,H,d] (Q, K, V = qkv[:, :, 0 / 1 / 2]).
+    Returns O as a [Z,H,N,d] view of memory laid out [Z,N,H,d].  Same arguments otherwise; the gradient of qkv comes
+    back as one tensor."""
+    if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
+        raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
+    if qkv.dim() != 5 or qkv.size(2) != 3:
+        raise AssertionError(f"qkv must be of shape (batch, N, 3, heads, d_k), not {tuple(qkv.shape)}")
+    if not _rows_ok(qkv[:, :, 0].permute(0, 2, 1, 3), qkv.element_size()):
+        qkv = qkv.contiguous()
+    return _geometric_attn_qkv.apply(qkv, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads, out_dtype, operand_dtype)
 
 
 def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00, max_rbf=1.00, check_spreads=True,
@@ -304,10 +353,10 @@ class GeoAttention(nn.Module):
 
         def heads_first(x):                # [Z, N, H*d_k] -> [Z, H, N, d_k] view
             return x.view(batch, N, H, dk).permute(0, 2, 1, 3)
+        qkv = None
         if q is k and k is v:
             w, b = self._fused_qkv()
-            qkv = torch.addmm(b, q.reshape(batch * N, d_model), w).view(batch, N, 3, H * dk)
-            Q, K, V = heads_first(qkv[:, :, 0]), heads_first(qkv[:, :, 1]), heads_first(qkv[:, :, 2])
+            qkv = torch.addmm(b, q.reshape(batch * N, d_model), w).view(batch, N, 3, H, dk)
         else:
             def flat(w_):                  # [H, d_model, d_k] -> [d_model, H*d_k]
                 return w_.permute(1, 0, 2).reshape(self.d_model, H * dk)
@@ -315,13 +364,14 @@ class GeoAttention(nn.Module):
             K = heads_first(torch.addmm(self.k_bias.reshape(-1), k.reshape(batch * N, d_model), flat(self.k_proj)))
             V = heads_first(torch.addmm(self.v_bias.reshape(-1), v.reshape(batch * N, d_model), flat(self.v_proj)))
         # sigma = min_spread + exp(w) is positive by construction: no need to read a check back from the device
-        if self.legacy_logits:
-            out = geometric_attn(Q, K, V, coords, self._per_head("spread"), self._per_head("beta"), mask=mask, min_rbf=self.min_rbf,
-                                 max_rbf=self.max_rbf, check_spreads=False, token_major_out=True, out_dtype=q.dtype,
-                                 operand_dtype=self.operand_dtype)
+        betas = self._per_head("beta") if self.legacy_logits else None
+        lo, hi = (self.min_rbf, self.max_rbf) if self.legacy_logits else (0.0, 1.0)
+        if qkv is not None:
+            out = geometric_attn_qkv(qkv, coords, self._per_head("spread"), betas, mask=mask, min_rbf=lo, max_rbf=hi,
+                                     check_spreads=False, out_dtype=q.dtype, operand_dtype=self.operand_dtype)
         else:
-            out = geometric_attn(Q, K, V, coords, self._per_head("spread"), None, mask=mask, check_spreads=False,
-                                 token_major_out=True, out_dtype=q.dtype)
+            out = geometric_attn(Q, K, V, coords, self._per_head("spread"), betas, mask=mask, min_rbf=lo, max_rbf=hi,
+                                 check_spreads=False, token_major_out=True, out_dtype=q.dtype, operand_dtype=self.operand_dtype)
         # The reference concatenates the heads as a (d_k x heads) interleave (encoder.py:114-115) before the output
         # projection.  Token-major O is the (heads x d_k) order; the same product is taken against the projection's
         # input columns in that order instead of reshuffling the activations.

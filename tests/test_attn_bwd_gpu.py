@@ -362,3 +362,40 @@ def test_delta_rowsum_equals_the_torch_expression(gpu, d, dtype):
     odd = torch.zeros(Z, H, N, d + 1)
     odd[..., 1:] = O
     check(_delta(odd.to(gpu)[..., 1:], dO.to(gpu)), "unaligned rows")
+
+
+@pytest.mark.parametrize("legacy", [False, True])
+def test_fused_projection_operator_equals_the_sliced_one(gpu, legacy):
+    """geometric_attn_qkv on qkv [Z,N,3,H,d] against geometric_attn on its three slices (what autograd then pads
+    and adds up): the same O, the same gradient of qkv to the bit (each element is one kernel result rounded once),
+    the per-head scalars to the rounding of their atomic sums."""
+    Z, H, N, d = 2, 3, 333, 64
+    g = torch.Generator().manual_seed(77)
+    base = torch.randn(Z, N, 3, H, d, generator=g).bfloat16()
+    dO = torch.randn(Z, H, N, d, generator=g).bfloat16().to(gpu)
+    coords = torch.stack([synth.random_walk_chain(N, g) for _ in range(Z)]).to(gpu)
+    sigma = torch.tensor([3.0, 7.0, 15.0])
+    betas = torch.tensor([0.3, 0.6, 1.1]) if legacy else None
+    lo, hi = (0.01, 0.98) if legacy else (0.0, 1.0)
+    mask = torch.zeros(Z, N, dtype=torch.bool)
+    mask[1, 300:] = True
+    res = []
+    for fused in (True, False):
+        qkv = base.clone().to(gpu).requires_grad_(True)
+        s = sigma.clone().to(gpu).requires_grad_(True)
+        b = None if betas is None else betas.clone().to(gpu).requires_grad_(True)
+        if fused:
+            O = pa.geometric_attn_qkv(qkv, coords, s, b, mask.to(gpu), lo, hi, out_dtype=torch.bfloat16)
+        else:
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            O = pa.geometric_attn(q, k, v, coords, s, b, mask.to(gpu), lo, hi, token_major_out=True, out_dtype=torch.bfloat16)
+        assert O.dtype == torch.bfloat16 and O.permute(0, 2, 1, 3).is_contiguous()
+        O.backward(dO)
+        res.append((O.detach(), qkv.grad, s.grad, None if b is None else b.grad))
+    (Oa, ga, sa, ba), (Ob, gb, sb, bb) = res
+    assert torch.equal(Oa, Ob)
+    assert ga.dtype == torch.bfloat16 and ga.shape == base.shape and torch.equal(ga, gb)
+    assert ga.abs().sum() > 0
+    assert torch.allclose(sa, sb, rtol=1e-4, atol=1e-7)
+    if legacy:
+        assert torch.allclose(ba, bb, rtol=1e-4, atol=1e-7)
