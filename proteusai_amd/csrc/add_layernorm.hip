@@ -153,7 +153,7 @@ extern "C" int proteus_add_layernorm_fwd_check(const void* x, const void* res, c
     if (!x || !out) return PROTEUS_ERR_NULL_POINTER;
     if (dtype != PROTEUS_DTYPE_F32 && dtype != PROTEUS_DTYPE_BF16) return PROTEUS_ERR_BAD_OPERAND_TYPE;
     const int vec = dtype == PROTEUS_DTYPE_F32 ? 4 : 8;
-    if (rows <= 0 || D <= 0 || rows > (1L << 31) * AL_WAVES - 1) return PROTEUS_ERR_BAD_SHAPE;
+    if (rows <= 0 || D <= 0 || rows > ((1L << 31) - 1) * AL_WAVES) return PROTEUS_ERR_BAD_SHAPE;      // grid.x below 2^31
     if (D % vec != 0 || D > 64 * vec * AL_MAX_CH) return PROTEUS_ERR_BAD_SHAPE;
     if (!(eps >= 0.0f)) return PROTEUS_ERR_BAD_SHAPE;
     const uintptr_t all = (uintptr_t)x | (uintptr_t)res | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)out;

@@ -88,6 +88,7 @@ int check(const float* O, const void* dO, const int64_t* strides, const float* D
     if (d_head != 32 && d_head != 64 && d_head != 128) return PROTEUS_ERR_BAD_HEAD_DIM;
     if (dtype != PROTEUS_DTYPE_F32 && dtype != PROTEUS_DTYPE_BF16 && dtype != PROTEUS_DTYPE_F16) return PROTEUS_ERR_BAD_OPERAND_TYPE;
     if (Z <= 0 || H <= 0 || N <= 0 || N > PROTEUS_ATTN_MAX_N || (long)Z * H > 65535) return PROTEUS_ERR_BAD_SHAPE;
+    if ((long)Z * H * N / (GD_THREADS / (d_head / 4)) >= (1L << 31) - 1) return PROTEUS_ERR_BAD_SHAPE;      // grid.x below 2^31
     const int gbytes = dtype == PROTEUS_DTYPE_F32 ? 4 : 2;
     if (((uintptr_t)O & 15) || ((uintptr_t)dO & (uintptr_t)(4 * gbytes - 1)) || ((uintptr_t)D & 3)) return PROTEUS_ERR_BAD_ALIGNMENT;
     if (!strides) {
