@@ -132,7 +132,7 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
 }
 
 // d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
-// the software-pipelined kernel runs (automatically for grids of at least 256 workgroups = one per CU, or when the tuning asks).
+// the software-pipelined kernel runs (automatically for large grids of long sequences, or when the tuning asks).
 int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords,
                 const float* sigma, const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
@@ -143,8 +143,14 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
     if (d_head == 128)
         return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 0 : tuning,
                                                beta, min_rbf, max_rbf, gs, st);
+    // The pipelined kernel pays a longer prologue back from about 16 key tiles per workgroup on, and only where its
+    // 256-query workgroups fill the chip twice: measured against the templated body it wins from 512 workgroups and
+    // N = 1024 on (3-11 %), loses below (7-9 % at 256 workgroups of N = 1024, 6-10 % at N = 256 and 512).  A batch that
+    // comes with a padding mask is taken to be ragged: up to N = 1024 such a batch runs 12-17 % faster on the body's
+    // 128-query workgroups (twice as many, half as long: they even out), so it goes there.
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
-    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 256)))
+    const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
+    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
         return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
     return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
