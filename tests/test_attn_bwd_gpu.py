@@ -125,6 +125,22 @@ def test_masks(gpu):
     compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "masks")
 
 
+def test_ragged_batch_of_long_sequences(gpu):
+    # N = 1024 (16 streamed tiles, 8 tiles of own tokens; a mask whose rows are multiples of 16 bytes): whole own tiles
+    # of padding, which leave without streaming anything, and sequences whose last unpadded token sits in the first,
+    # a middle and the last tile, where the streaming stops; one item padded in the middle only.
+    N = 1024
+    Q, K, V, dO, coords, sigma, _ = make(7, 6, 2, N)
+    mask = torch.zeros(6, N, dtype=torch.bool)
+    mask[1, 700:] = True
+    mask[2, 130:] = True
+    mask[3, 64:] = True
+    mask[4, 1:] = True
+    mask[5, 300:600] = True
+    a = (Q, K, V, dO, coords, sigma, mask)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "ragged N=1024")
+
+
 def test_padded_content_cannot_matter(gpu):
     Q, K, V, dO, coords, sigma, mask = make(2, 2, 4, 260, maskfrac=0.3)
     got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask)
