@@ -392,6 +392,24 @@ def main():
                             "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
                             "frac": useful / (ms3 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
                             "flop": "4 H d sum_b L_b^2 (pairs of valid tokens only)"}}
+        # the backward of the same padded batch (kernel call only: D precomputed; d_sigma accumulates, it is not read)
+        attn_forward_into(q3, k3, v3, c3d, s3d, m3d, O3, L3)
+        g3 = torch.Generator().manual_seed(3)
+        dO3 = (torch.randn(4, 8, 4096, 64, generator=g3) / 8).bfloat16().to(dev)
+        D3 = (O3 * dO3.float()).sum(-1).contiguous()
+        dQ3, dK3, dV3 = (torch.empty(4, 8, 4096, 64, device=dev) for _ in range(3))
+        ds3 = torch.zeros(8, device=dev)
+
+        def bwd3_step():
+            rc = lib.proteus_geo_attn_bwd(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), dO3.data_ptr(), c3d.data_ptr(), s3d.data_ptr(),
+                                          None, m3d.data_ptr(), L3.data_ptr(), D3.data_ptr(), dQ3.data_ptr(), dK3.data_ptr(), dV3.data_ptr(),
+                                          ds3.data_ptr(), None, 4, 8, 4096, 64, 0.0, 1.0, _lib.OPERAND_BF16, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_geo_attn_bwd")
+        _, bms3 = time_launches(torch, bwd3_step, 20)
+        leg["backward_ms"] = bms3
+        leg["backward_tflops_useful_5_products"] = 2.5 * useful / (bms3 * 1e-3) / 1e12
+        del dO3, D3, dQ3, dK3, dV3
         if not args.no_cpu:
             dt, runs = cpu_timed(lambda: torch_oracle.geo_attn_torch(Q3, K3, V3, c3, sg3, m3), 20.0, 3)
             leg["cpu_baseline"] = {"value": dense / dt / 1e12, "unit": "TFLOP/s (dense-equivalent: the CPU path computes every pair and masks)",
