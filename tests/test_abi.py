@@ -184,6 +184,22 @@ def test_operator_argument_errors_match_the_reference_surface():
         pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), None, min_rbf=0.1)     # the pair mask needs betas
     with pytest.raises(_lib.ProteusError):
         pa.geometric_attn(Q, Q, Q, coords, torch.ones(2), betas=torch.ones(2))    # legacy logits exist, but not on the CPU
+    # the operator on a fused projection: qkv is [Z,N,3,H,d]
+    qkv = torch.randn(1, 8, 3, 2, 64)
+    with pytest.raises(AssertionError):
+        pa.geometric_attn_qkv(qkv[:, :, :2], coords, torch.ones(2))
+    with pytest.raises(AssertionError):
+        pa.geometric_attn_qkv(qkv[0], coords, torch.ones(2))
+    with pytest.raises(NotImplementedError):
+        pa.geometric_attn_qkv(qkv, coords, torch.ones(2), None, max_rbf=0.9)
+    with pytest.raises(_lib.ProteusError):
+        pa.geometric_attn_qkv(qkv, coords, torch.ones(2))                         # not on the CPU
+    # the encoder layer's add + LayerNorm falls back to the torch expression wherever the kernel does not apply (CPU here)
+    from proteusai_amd.encoder import add_layer_norm
+    norm = torch.nn.LayerNorm(16)
+    x, r = torch.randn(3, 16), torch.randn(3, 16)
+    with torch.no_grad():
+        assert torch.equal(add_layer_norm(x, r, norm), norm(x + r))
 
 
 def test_wavefunction_embedding_module_schedule_and_parameters():
