@@ -194,7 +194,8 @@ def test_operator_argument_errors_match_the_reference_surface():
         pa.geometric_attn_qkv(qkv, coords, torch.ones(2), None, max_rbf=0.9)
     with pytest.raises(_lib.ProteusError):
         pa.geometric_attn_qkv(qkv, coords, torch.ones(2))                         # not on the CPU
-    # the encoder layer's add + LayerNorm falls back to the torch expression wherever the kernel does not apply (CPU here)
+    # the encoder layer's add + LayerNorm is the torch expression itself for tensors the kernel does not take (CPU tensors here;
+    # the two O(N^2) operators around it have no CPU path and raise)
     from proteusai_amd.encoder import add_layer_norm
     norm = torch.nn.LayerNorm(16)
     x, r = torch.randn(3, 16), torch.randn(3, 16)
