@@ -476,7 +476,12 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
             const double cs = w <= 1 ? 4.8 : (w == 2 ? 4.15 : 4.0);
             const double ct = w <= 1 ? 10.3 : (w == 2 ? 9.0 : 8.3);
             const double per_wave = keys * (ckt * (cs + 2.0 * ct + 4.0 * cv) + 15.0 * cv + ct + 30.0);
-            const double est = (q > w ? q : (double)w) * per_wave;
+            double est = (q > w ? q : (double)w) * per_wave;
+            // A batch that comes with a padding mask is taken to be ragged.  While the widest tile gives at most 1024
+            // workgroups (little more than one round of the chip), halving the tile makes twice as many workgroups of
+            // half the length, which even out better than the wider tile saves: 8 x 1024 with lengths 128-1024 runs
+            // 5-30 % faster (six draws of the lengths), the same batch without padding 2 % slower.
+            if (mask && ckt == 32 && csp && nwaves <= 4096) est *= 1.10;
             if (est < best * 0.999) { best = est; kt = ckt; split = csp; }
         }
     }
