@@ -396,7 +396,7 @@ extern "C" int proteus_we_aniso_fwd(const float* coordsA, const float* coordsB, 
         const long ktiles  = ((long)K + kt - 1) / kt;
         double best = 1e300;
         for (int csp = 1; csp >= 0; --csp) {
-            if (csp && N < 4 * 64) continue;
+            if (csp && N < 2 * WA_WAVES) continue;          // (fewer sources than a split could share out)
             const long nwaves = csp ? iblocks * ktiles * WA_WAVES : iblocks * ((ktiles + WA_WAVES - 1) / WA_WAVES) * WA_WAVES;
             const double keys = csp ? (double)N / WA_WAVES : (double)N;
             const double rounds = (double)((nwaves + 1023) / 1024);

@@ -400,6 +400,7 @@ const WeVariant kVariants[] = {
     {"kt32_split", 32, true, 0},
     {"kt32_fract", 32, false, 1},
     {"kt32_nofract_unchecked", 32, false, -1},
+    {"kt4_split", 4, true, 0},
 };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
@@ -459,14 +460,14 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
         // (clocks per wave instruction, measured: vector-operand 5.8 / 2.9 / 2.5, scalar-operand
         // 4.8 / 4.15 / 4.0, transcendental 10.3 / 9.0 / 8.3 with 1 / 2 / 3+ waves).  `occ` is what the
         // kernel's registers allow.  Ties keep the earlier candidate.
-        static const int cand_kt[6]    = {32, 32, 16, 16, 8, 8};
-        static const int cand_split[6] = {1, 0, 1, 0, 1, 0};
-        static const int cand_occ[6]   = {3, 2, 4, 4, 8, 8};
+        static const int cand_kt[7]    = {32, 32, 16, 16, 8, 8, 4};
+        static const int cand_split[7] = {1, 0, 1, 0, 1, 0, 1};
+        static const int cand_occ[7]   = {3, 2, 4, 4, 8, 8, 8};
         double best = 1e300;
-        for (int c = 0; c < 6; ++c) {
+        for (int c = 0; c < 7; ++c) {
             const int  ckt = cand_kt[c];
             const bool csp = cand_split[c] != 0;
-            if (csp && N < 4 * 64) continue;
+            if (csp && N < 2 * WE_WAVES) continue;          // (fewer sources than a split could share out)
             const long ktiles = ((long)K + ckt - 1) / ckt;
             const long nwaves = csp ? iblocks * ktiles * WE_WAVES : iblocks * ((ktiles + WE_WAVES - 1) / WE_WAVES) * WE_WAVES;
             const double keys = csp ? (double)N / WE_WAVES : (double)N;
@@ -492,6 +493,7 @@ extern "C" int proteus_we_fwd(const float* coords, int coords_layout,
     switch (kt) {
         case 32: return WE_GO(32);
         case 16: return WE_GO(16);
+        case 4:  return WE_GO(4);
         default: return WE_GO(8);
     }
 #undef WE_GO
