@@ -330,7 +330,7 @@ def main():
         _, ms1 = time_launches(torch, lambda: we_forward_into(c1d, w, None, o1, cs1, ss1), 200)
         W1 = 512.0 * 512 * K
         leg = {"workload": "WE forward B=1 N=512 d_model=512, random-walk chain, no mask (BASELINE.json configs[0]); "
-                           "8 observer blocks of 64 rows x 4 wavenumber slices: 32 workgroups on 256 CUs, a launch-latency-sized kernel",
+                           "8 observer blocks of 64 rows x 64 tiles of 4 wavenumbers: 512 short workgroups, a launch-latency-sized kernel",
                "ms": ms1, "gpair_wavenumber_per_s": W1 / (ms1 * 1e-3) / 1e9, "dtype": "f32",
                "roofline": {"kernel": "we_fwd_kernel", "bound": "valu", "achieved": 9.0 * W1 / (ms1 * 1e-3) / 1e12,
                             "peak": PEAK_FP32_VECTOR_TFLOPS, "unit": "TFLOP/s",
