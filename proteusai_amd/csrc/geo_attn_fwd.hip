@@ -79,7 +79,7 @@ static_assert(GA_PIPE_LDS <= 80 * 1024, "two workgroups per compute unit");
 
 struct GaVariant { const char* name; };
 const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"},
-                                {"pipelined"}, {"pipelined_dist_mfma"} };
+                                {"pipelined"}, {"pipelined_dist_mfma"}, {"split_keys"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -138,10 +138,10 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
 {
     if (d_head == 32)
-        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 0 : tuning,
+        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 0 : tuning,
                                               beta, min_rbf, max_rbf, gs, st);
     if (d_head == 128)
-        return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 0 : tuning,
+        return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 0 : tuning,
                                                beta, min_rbf, max_rbf, gs, st);
     // The pipelined kernel pays a longer prologue back from about 16 key tiles per workgroup on, and only where its
     // 256-query workgroups fill the chip twice: measured against the templated body it wins from 512 workgroups and
@@ -152,7 +152,7 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
     const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
     if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
         return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
-    return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning >= 5 ? 4 : tuning,
+    return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
 }
 // contiguous [Z,H,N,d] tensors
