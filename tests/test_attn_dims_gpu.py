@@ -61,7 +61,7 @@ def check_forward(O, L, Q, K, V, coords, sigma, mask, betas, lo, hi, lse_tol, wh
 @pytest.mark.parametrize("N", [1, 33, 64, 130, 257, 600])
 def test_forward_readme_logits(gpu, d, N):
     Q, K, V, _, coords, sigma, mask = make(500 + N + d, 2, 3, N, d, torch.bfloat16, maskfrac=0.2 if N > 33 else 0.0)
-    for tuning in (0, 1, 2, 3, 4):          # automatic; matrix-core / direct distances; one / two query blocks per wave
+    for tuning in (0, 1, 2, 3, 4, 7):       # automatic; matrix-core / direct distances; one / two query blocks per wave; keys split
         O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), None if mask is None else mask.to(gpu),
                            return_lse=True, tuning=tuning)
         check_forward(O, L, Q, K, V, coords, sigma, mask, None, 0.0, 1.0, LSE_TOL_BF16, f"d={d} N={N} tuning={tuning}")

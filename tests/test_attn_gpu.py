@@ -45,7 +45,7 @@ def make(seed, Z, H, N, qscale=1.0, maskfrac=0.0, tail=False):
 
 # 0: the launcher's choice (small grids take the kernel with one query block per wave); 5: the software-pipelined
 # kernel, which large grids take, forced on these small shapes too (its direct-distance fallback beside it)
-KERNELS = [0, 5]
+KERNELS = [0, 3, 5, 7]      # automatic; one query block per wave; the pipelined kernel; a pair of waves per query block (keys split)
 
 
 def run_gpu(gpu, Q, K, V, coords, sigma, mask, tuning=0):
