@@ -115,6 +115,55 @@ def probe_rates(lib, torch, dev):
     return rates
 
 
+def probe_trans_valu_overlap(lib, torch, dev, waves_per_simd=3, blocks=256):
+    """Do transcendental and ordinary vector instructions of different waves of one SIMD overlap?
+
+    One workgroup per compute unit, `waves_per_simd` waves on every SIMD (the headline kernel's occupancy), k of them
+    issuing only v_sin_f32 chains and the others only v_fmac_f32 chains with vector-register operands; iteration counts
+    chosen so that either group alone takes about the same time.  Returns per k: the two times alone, the time
+    together, and hidden = (alone_t + alone_v - together) / min(alone_t, alone_v): 0 = they take turns, 1 = the shorter
+    runs entirely beside the longer.  The placement (waves_per_simd waves of a workgroup on each SIMD) is read back
+    from the hardware-id register and reported."""
+    sink = torch.empty(blocks * 256 * waves_per_simd, device=dev)
+    census = torch.zeros(blocks * 4, dtype=torch.int32, device=dev)
+
+    def run(k, it_t, it_v):
+        def go():
+            rc = lib.proteus_probe_trans_valu_mix(waves_per_simd, k, blocks, it_t, it_v, sink.data_ptr(), census.data_ptr(), None)
+            assert rc == 0, rc
+        go()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            go()
+            e1.record()
+            torch.cuda.synchronize()
+            best = e0.elapsed_time(e1) if best is None else min(best, e0.elapsed_time(e1))
+        return best
+
+    out = {"waves_per_simd": waves_per_simd}
+    base = 4000
+    for k in range(1, waves_per_simd):
+        # calibrate: links of the ordinary group so that it takes as long alone as the transcendental group alone
+        t_alone = run(k, base, 0)
+        v_probe = run(k, 0, base)
+        it_v = max(1, int(base * t_alone / v_probe))
+        v_alone = run(k, 0, it_v)
+        both = run(k, base, it_v)
+        cen = census.cpu().numpy().astype("int64")
+        placed_ok = bool(((cen >> 16) == waves_per_simd).all() and ((cen & 0xffff) == k).all())
+        out[f"k{k}"] = {
+            "trans_waves": k, "valu_waves": waves_per_simd - k, "trans_alone_ms": t_alone, "valu_alone_ms": v_alone,
+            "together_ms": both, "hidden": (t_alone + v_alone - both) / min(t_alone, v_alone),
+            "placement_as_assumed": placed_ok,
+            "lane_ops_per_s_together": {"transcendental": blocks * 4 * k * 64.0 * base * 64 / (both * 1e-3),
+                                        "ordinary": blocks * 4 * (waves_per_simd - k) * 64.0 * it_v * 64 / (both * 1e-3)},
+        }
+    return out
+
+
 def probe_slot_ms(lib, torch, dev, mode, blocks=512, iters=4000):
     """Seconds per slot per SIMD of the co-issue probe (a slot = one 32x32x16 bf16 product + the softmax work of two
     scores) at two waves per SIMD: blocks x 4 waves x iters x 8 slots over 1024 SIMDs."""
@@ -155,8 +204,9 @@ def main():
         sys.exit(2)
 
     import torch
-    from proteusai_amd import _lib, synth
+    from proteusai_amd import _lib, _probes, synth
     lib = _lib.load()
+    probes = _probes.load()                   # measurement-only library (instruction rates, co-issue); not the product
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
@@ -205,7 +255,7 @@ def main():
     W = float(Z) * N * N * K                          # pair*wavenumber evaluations per step
     value = W * args.steps / elapsed / 1e9            # Gpair*wavenumber/s, whole job
 
-    rates = probe_rates(lib, torch, dev)
+    rates = probe_rates(probes, torch, dev)
     # per unit: the phase product (scalar operand), v_sin, v_cos, two v_fmac and two v_add on vector operands
     r_trans = (rates["sin"] + rates["cos"]) / 2
     per_unit_s = 1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / rates["add_v"] + 2.0 / r_trans
@@ -229,6 +279,25 @@ def main():
         "vendor_rate_model": {"lane_ops_per_s": {"ordinary": 3.93e13, "transcendental": 9.83e12},
                               "model_ms": W * (5.0 / 3.93e13 + 2.0 / 9.83e12) * 1e3,
                               "frac": W * (5.0 / 3.93e13 + 2.0 / 9.83e12) * 1e3 / avg_kernel_ms},
+    }
+    # the published 157.3 TFLOP/s counts packed (two-wide) fp32 FMAs, which this build never issues; beside it the
+    # fraction of the one-wide vector rate, half of it
+    roofline["peak_non_packed"] = PEAK_FP32_VECTOR_TFLOPS / 2
+    roofline["frac_of_non_packed_peak"] = achieved_tflops / (PEAK_FP32_VECTOR_TFLOPS / 2)
+    # The issue model adds the transcendentals' time to the ordinary instructions' time.  Whether the two kinds, issued
+    # by different waves of a SIMD, run beside each other is measured here; if they did, the bound would be the larger
+    # of the two times instead of their sum.
+    t_ord_ms = W * (1.0 / rates["mul_s"] + 2.0 / rates["fmac_v"] + 2.0 / rates["add_v"]) * 1e3
+    t_trn_ms = W * (2.0 / r_trans) * 1e3
+    overlap = probe_trans_valu_overlap(probes, torch, dev)
+    hidden = min(v["hidden"] for k_, v in overlap.items() if k_.startswith("k"))
+    hidden = max(0.0, min(1.0, hidden))
+    bound_ms = t_ord_ms + t_trn_ms - hidden * min(t_ord_ms, t_trn_ms)
+    roofline["issue_model"]["trans_valu_overlap"] = {
+        "probe": overlap, "hidden_fraction_used": hidden,
+        "ordinary_ms": t_ord_ms, "transcendental_ms": t_trn_ms,
+        "model_ms_with_measured_overlap": bound_ms, "frac_with_measured_overlap": bound_ms / avg_kernel_ms,
+        "model_ms_if_fully_overlapped": max(t_ord_ms, t_trn_ms), "frac_if_fully_overlapped": max(t_ord_ms, t_trn_ms) / avg_kernel_ms,
     }
     pw = read_profile(PROFILE_WE)
     if "valu_insts_per_unit" in pw:
@@ -440,7 +509,7 @@ def main():
         # scores, 4 for P V), each with the softmax work of two scores per lane.  The probe measures what one SIMD needs per
         # slot at the kernel's occupancy (two waves) when it does nothing else: no staging, no geometry, no barrier.
         slots = 8.0 * 8 * (16384 / 32) * (16384 / 32) / 1024.0               # per SIMD
-        t_m, t_v, t_b = (probe_slot_ms(lib, torch, dev, m) for m in (0, 1, 2))
+        t_m, t_v, t_b = (probe_slot_ms(probes, torch, dev, m) for m in (0, 1, 2))
         leg["roofline"]["issue_model"] = {
             "slot": "one 32x32x16 bf16 product + 2 fma + 2 exp2 + 1 pack + 1 packed add, two waves per SIMD",
             "ns_per_slot_per_simd": {"matrix_only": t_m * 1e9, "vector_only": t_v * 1e9, "both": t_b * 1e9},
@@ -449,7 +518,7 @@ def main():
         }
         # which vector instructions run beside a matrix product: the same loop with the softmax work replaced by
         # twelve ordinary fused multiply-adds, and by four exp2 (ns per slot and SIMD: alone, and with the product)
-        t_pa, t_pm, t_ta, t_tm = (probe_slot_ms(lib, torch, dev, m) for m in (3, 4, 5, 6))
+        t_pa, t_pm, t_ta, t_tm = (probe_slot_ms(probes, torch, dev, m) for m in (3, 4, 5, 6))
         leg["roofline"]["issue_model"]["beside_a_product_ns"] = {
             "twelve_fma": {"alone": t_pa * 1e9, "with_product": t_pm * 1e9, "hidden_frac": (t_m + t_pa - t_pm) / t_pa},
             "four_exp2": {"alone": t_ta * 1e9, "with_product": t_tm * 1e9, "hidden_frac": (t_m + t_ta - t_tm) / t_ta},

@@ -59,7 +59,14 @@ extern "C" {
 #define PROTEUS_ATTN_MAX_N (1 << 20)
 #define PROTEUS_WE_BWD_STATIC_MAX_K 512   /* most wavenumbers proteus_we_bwd_static takes */
 
-/* Library version (major*10000 + minor*100 + patch). */
+/*
+ * Library version (major*10000 + minor*100 + patch) as a number that only grows.  PROTEUS_VERSION is the version this
+ * header describes; a caller built against it should refuse a library whose proteus_version() differs in
+ * major*10000 + minor*100 (argument lists have changed between minors: since 210 the beta-weighted forward and every
+ * backward entry point take `int operand_type` before `tuning` / `stream`; a caller built against an older header
+ * would pass its tuning selector there).  The Python binding checks for an exact match when it loads the library.
+ */
+#define PROTEUS_VERSION 300
 int proteus_version(void);
 
 /* Human-readable text for a return code of any entry point. */
@@ -203,6 +210,9 @@ int proteus_we_bwd_check(const float* d_out, const float* cos_sums, const float*
  *   The GPU that is current at the call must be the one `stream` belongs to.
  *   All calls on one GPU share that GPU's array: calls that overlap there (two
  *   streams, two threads) race; serialise them.  Nothing has to be cleared between calls.
+ *   The first call made with a given GPU current looks the array's address up (hipGetSymbolAddress, under a mutex)
+ *   and may load the library's device image: make that first call per GPU outside stream capture; every later call
+ *   only launches its two kernels and can be captured.
  */
 int proteus_we_bwd_static(const float* d_out, const float* cos_sums, const float* sin_sums,
                           float* d_wavenumbers, int Z, int N, int K, void* stream);
@@ -384,40 +394,6 @@ int proteus_add_layernorm_fwd(const void* x, const void* res, const void* gamma,
                               long rows, int D, float eps, int dtype, void* stream);
 int proteus_add_layernorm_fwd_check(const void* x, const void* res, const void* gamma, const void* beta, const void* out,
                                     long rows, int D, float eps, int dtype);
-
-/*
- * Instruction-rate probe used to state the roofline denominator of the WE
- * kernel.  Runs `iters` rounds of 64 independent chains of one VALU
- * instruction per lane on `blocks` x 256 threads and writes one float per
- * thread to `sink` (blocks * 256 floats; so the work cannot be removed).  The
- * caller times the launch; lane-ops issued = blocks*256*iters*64.  No
- * counterpart in the reference.
- *   op: 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32 (second operand a scalar register),
- *       3 v_sin_f32, 4 v_cos_f32, 5 v_exp_f32, 6 v_rsq_f32, 7 v_fract_f32;
- *       8 v_fmac_f32 and 9 v_add_f32 with vector-register operands only.
- */
-int proteus_probe_valu_rate(int op, int blocks, int iters, float* sink, void* stream);
-
-/*
- * Accuracy probe of the hardware sin/cos path used by the WE kernel:
- * s[i] = v_sin_f32(y), c[i] = v_cos_f32(y) with x in revolutions and
- * y = fract(x[i]) if use_fract else x[i] (the instructions accept |y| <= 256),
- * and q[i] = refined sqrt path r = r2*rsq(r2) applied to x[i].
- */
-int proteus_probe_sincos(const float* x, float* s, float* c, float* q, int n, int use_fract, void* stream);
-
-/*
- * Co-issue probe behind the attention forward's issue model (no counterpart in the reference).  Every wave runs
- * `iters` loop trips of eight "slots"; a slot is what the attention kernel's inner loop issues per 32x32x16 bf16
- * matrix product: that product and the softmax work of two scores (2 fused multiply-adds, 2 exp2, 1 pack to bf16,
- * 1 packed row-sum add).  mode 0: the matrix products only; 1: the vector work only; 2: both.  Modes 3-6 replace
- * the vector work, to tell which kind of vector instruction runs beside a matrix product: 3: twelve ordinary fused
- * multiply-adds per slot, alone; 4: those with the products; 5: four exp2 per slot, alone; 6: those with the
- * products.  `blocks`
- * workgroups of 256 threads (512 on a 256-CU chip = two waves per SIMD, the attention kernel's occupancy);
- * sink [blocks*256] f32 receives values that keep the work alive.  Time the launch with events.
- */
-int proteus_probe_mfma_softmax_slot(int mode, int blocks, int iters, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "libproteus_hip.so")
 
 COORDS_SOA = 0
 COORDS_AOS = 1
+ABI_VERSION = 300                    # PROTEUS_VERSION of the include/proteus_hip.h these argument lists were written from
 OPERAND_BF16, OPERAND_F16 = 0, 1     # PROTEUS_OPERAND_* of include/proteus_hip.h
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2   # PROTEUS_DTYPE_*
 
@@ -26,7 +27,6 @@ SYMBOLS = [
     "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
     "proteus_geo_attn_variant_name",
     "proteus_add_layernorm_fwd", "proteus_add_layernorm_fwd_check", "proteus_geo_attn_delta", "proteus_geo_attn_delta_check",
-    "proteus_probe_valu_rate", "proteus_probe_sincos", "proteus_probe_mfma_softmax_slot",
 ]
 
 _lib = None
@@ -48,6 +48,9 @@ def load():
     lib = ctypes.CDLL(LIB_PATH)
     vp, ci = ctypes.c_void_p, ctypes.c_int
     lib.proteus_version.restype = ci
+    if lib.proteus_version() != ABI_VERSION:
+        raise ProteusError(f"{LIB_PATH} reports version {lib.proteus_version()}, this binding was written for {ABI_VERSION}: "
+                           "argument lists differ between versions; rebuild with `python -m proteusai_amd.build`")
     lib.proteus_strerror.restype = ctypes.c_char_p
     lib.proteus_strerror.argtypes = [ci]
     lib.proteus_we_fwd.restype = ci
@@ -114,12 +117,6 @@ def load():
     lib.proteus_geo_attn_delta.argtypes = [vp, vp, i64p, vp, ci, ci, ci, ci, ci, vp]
     lib.proteus_geo_attn_delta_check.restype = ci
     lib.proteus_geo_attn_delta_check.argtypes = [vp, vp, i64p, vp, ci, ci, ci, ci, ci]
-    lib.proteus_probe_valu_rate.restype = ci
-    lib.proteus_probe_valu_rate.argtypes = [ci, ci, ci, vp, vp]
-    lib.proteus_probe_sincos.restype = ci
-    lib.proteus_probe_sincos.argtypes = [vp, vp, vp, vp, ci, ci, vp]
-    lib.proteus_probe_mfma_softmax_slot.restype = ci
-    lib.proteus_probe_mfma_softmax_slot.argtypes = [ci, ci, ci, vp, vp]
     _lib = lib
     return lib
 

@@ -1,4 +1,5 @@
-"""Compile the HIP sources under csrc/ into proteusai_amd/libproteus_hip.so for gfx950.
+"""Compile the HIP sources under csrc/ into proteusai_amd/libproteus_hip.so for gfx950, and the measurement probes
+(csrc/probes.hip, which the benchmark and one test load, nothing else) into proteusai_amd/libproteus_probes.so.
 
 Plain `hipcc -shared -fPIC`; no torch extension machinery (the library has a C
 ABI and is loaded with ctypes).  hipcc cross-compiles without a GPU present.
@@ -12,7 +13,9 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "libproteus_hip.so")
 SOURCES = ["abi.hip", "we_fwd.hip", "we_aniso_fwd.hip", "we_bwd.hip", "geo_attn_fwd.hip", "geo_attn_fwd_d32.hip", "geo_attn_fwd_d128.hip",
-           "geo_attn_bwd.hip", "geo_attn_bwd_d32.hip", "geo_attn_bwd_d128.hip", "geo_attn_delta.hip", "add_layernorm.hip", "probe.hip"]
+           "geo_attn_bwd.hip", "geo_attn_bwd_d32.hip", "geo_attn_bwd_d128.hip", "geo_attn_delta.hip", "add_layernorm.hip"]
+PROBE_LIB = os.path.join(HERE, "libproteus_probes.so")
+PROBE_SOURCES = ["probes.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -28,11 +31,11 @@ FLAGS = [
 
 
 def build(verbose: bool = False) -> str:
-    """Compile every source (always; no up-to-date check) and link the library."""
+    """Compile every source (always; no up-to-date check) and link the two libraries.  Returns the product library."""
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
-    for src in SOURCES:
+    for src in SOURCES + PROBE_SOURCES:
         obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
         cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
@@ -50,8 +53,9 @@ def build(verbose: bool = False) -> str:
             print("\n".join(lines))
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
-    subprocess.run(cmd, check=True)
+    n = len(SOURCES)
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs[:n], check=True)
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB] + objs[n:], check=True)
     return LIB
 
 

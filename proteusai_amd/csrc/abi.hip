@@ -3,7 +3,7 @@
 #include <hip/hip_runtime.h>
 #include "proteus_hip.h"
 
-extern "C" int proteus_version(void) { return 210; }
+extern "C" int proteus_version(void) { return PROTEUS_VERSION; }
 
 extern "C" const char* proteus_strerror(int code) {
     switch (code) {

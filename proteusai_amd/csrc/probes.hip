@@ -4,7 +4,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include "proteus_hip.h"
+#include "proteus_hip.h"      // return codes
+#include "proteus_probes.h"
 
 namespace {
 
@@ -138,7 +139,70 @@ void mfma_softmax_slot_kernel(float* sink, int iters) {
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// Do transcendental and ordinary vector instructions of DIFFERENT waves of one SIMD overlap?  One workgroup of
+// 4 * WPS waves per compute unit (its LDS request keeps a second one away), WPS waves on every SIMD.  Each wave reads
+// the SIMD it runs on from the hardware-id register and draws a ticket among the waves of its workgroup on that SIMD:
+// the first `k_trans` tickets run `iters_trans` links of 64 independent v_sin_f32 chains, the others `iters_valu`
+// links of 64 independent v_fmac_f32 chains with vector-register operands only.  census[workgroup * 4 + simd] receives
+// (waves seen << 16) | waves that took the transcendental role, so the host can check the placement it relies on.
+__global__ __launch_bounds__(1024)
+void trans_valu_mix_kernel(float* sink, unsigned* census, int k_trans, int iters_trans, int iters_valu, float a, float b) {
+    extern __shared__ unsigned mix_lds[];            // [0..3]: tickets per SIMD, [4..7]: transcendental waves per SIMD
+    if (threadIdx.x < 8) mix_lds[threadIdx.x] = 0u;
+    __syncthreads();
+    // HW_REG_HW_ID (register 4), bits 5:4 = SIMD_ID
+    const unsigned simd = __builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4) & 3u;
+    unsigned ticket = 0;
+    if ((threadIdx.x & 63) == 0) ticket = atomicAdd(&mix_lds[simd], 1u);
+    ticket = (unsigned)__builtin_amdgcn_readfirstlane((int)ticket);
+    const bool trans = (int)ticket < k_trans;
+    if (trans && (threadIdx.x & 63) == 0) atomicAdd(&mix_lds[4 + simd], 1u);
+    float x[64];
+#pragma unroll
+    for (int c = 0; c < 64; ++c) x[c] = 0.001f * (float)((threadIdx.x & 63) + c) + 0.25f;
+    float u = 1e-3f * (a + 1e-9f * (float)threadIdx.x), v = b + 1e-12f * (float)threadIdx.x;
+    if (trans) {
+#pragma unroll 1
+        for (int it = 0; it < iters_trans; ++it) {
+#pragma unroll
+            for (int c = 0; c < 64; ++c) x[c] = __builtin_amdgcn_sinf(x[c]);
+        }
+    } else {
+#pragma unroll 1
+        for (int it = 0; it < iters_valu; ++it) {
+#pragma unroll
+            for (int c = 0; c < 64; ++c) x[c] = __builtin_fmaf(u, v, x[c]);
+            asm volatile("" : "+v"(u), "+v"(v));
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 64; ++c) s += x[c];
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x < 4) census[blockIdx.x * 4 + threadIdx.x] = (mix_lds[threadIdx.x] << 16) | mix_lds[4 + threadIdx.x];
+}
+
 }  // namespace
+
+extern "C" int proteus_probe_trans_valu_mix(int waves_per_simd, int k_trans, int blocks, int iters_trans, int iters_valu,
+                                            float* sink, unsigned* census, void* stream) {
+    if (!sink || !census) return PROTEUS_ERR_NULL_POINTER;
+    if (blocks <= 0 || blocks > (1 << 20) || iters_trans < 0 || iters_valu < 0) return PROTEUS_ERR_BAD_SHAPE;
+    if (waves_per_simd < 1 || waves_per_simd > 4 || k_trans < 0 || k_trans > waves_per_simd) return PROTEUS_ERR_BAD_TUNING;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // 96 KB of LDS per workgroup: one workgroup per compute unit (160 KB each)
+    static bool allowed = false;
+    if (!allowed) {
+        const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(trans_valu_mix_kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        if (attr != hipSuccess) return (int)attr;
+        allowed = true;
+    }
+    hipLaunchKernelGGL(trans_valu_mix_kernel, dim3(blocks), dim3(256 * waves_per_simd), 96 * 1024, st,
+                       sink, census, k_trans, iters_trans, iters_valu, 0.999999f, 1e-7f);
+    return (int)hipGetLastError();
+}
 
 extern "C" int proteus_probe_mfma_softmax_slot(int mode, int blocks, int iters, float* sink, void* stream) {
     if (!sink) return PROTEUS_ERR_NULL_POINTER;

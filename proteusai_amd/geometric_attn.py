@@ -233,6 +233,11 @@ class _geometric_attn(torch.autograd.Function):
                 None if betas is None else d_beta.to(betas.dtype), None, None, None, None, None, None, None)
 
 
+def _fused_grad_views_ok(grads):
+    """Can the backward kernels write dQ, dK, dV straight into these views of one fused [Z,N,3,H,d] fp32 buffer?"""
+    return all(_rows_ok(g_, 4) for g_ in grads)
+
+
 class _geometric_attn_qkv(torch.autograd.Function):
     """The same operator on a fused projection qkv [Z,N,3,H,d] (self-attention: what one GEMM over the three
     projections leaves).  Forward and backward read Q, K, V in place; the backward writes dQ, dK, dV into one
@@ -254,8 +259,16 @@ class _geometric_attn_qkv(torch.autograd.Function):
         Q, K, V = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         g = torch.empty(qkv.shape, dtype=torch.float32, device=qkv.device)
         grads = tuple(g[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-        _, _, _, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
-                                                     ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype, grads=grads)
+        if _fused_grad_views_ok(grads):
+            _, _, _, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
+                                                         ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype, grads=grads)
+        else:
+            # a sequence of the fused buffer spans 2 GiB or more: the kernels cannot address it in place, so the
+            # gradients go to buffers of their own (as the sliced operator does) and are copied in
+            dQ, dK, dV, d_sigma, d_beta = geo_attn_backward(Q, K, V, O, L, dO, coords, spreads, mask, betas,
+                                                            ctx.min_rbf, ctx.max_rbf, ctx.operand_dtype)
+            for dst, src in zip(grads, (dQ, dK, dV)):
+                dst.copy_(src)
         return (g.to(qkv.dtype), None, d_sigma.to(spreads.dtype), None if betas is None else d_beta.to(betas.dtype),
                 None, None, None, None, None, None)
 
@@ -378,12 +391,42 @@ class GeoAttention(nn.Module):
         out = out.permute(0, 2, 1, 3).reshape(batch, N, self.d_model)           # a view when O is token-major
         return torch.nn.functional.linear(out, self._out_weight())
 
+    # ---- constants derived from the parameters, kept across inference calls ----
+    # sigma / beta of the heads, the output projection with its columns permuted and the fused projection weight are
+    # functions of the parameters.  They are kept across calls only in eval() mode and only where no gradient is
+    # needed, keyed on the parameters' version counters and storage, and dropped by anything that is known to change
+    # the weights: train() / eval(), .to() / .half() / .cuda() (through _apply), load_state_dict, and
+    # invalidate_caches().  A write through `p.data` (e.g. `p.data.copy_(ema)`) bumps no version counter and cannot be
+    # seen from here: after such a write in eval() mode call invalidate_caches() (or eval() again).
+
+    def invalidate_caches(self):
+        """Drop the constants kept from earlier inference calls.  Needed only after the parameters were changed
+        behind autograd's back (writes through `.data`) while the module stayed in eval() mode."""
+        self.__dict__.pop("_head_cache", None)
+        self._wo_cache = None
+        self._qkv_cache = None
+
+    def train(self, mode: bool = True):
+        self.invalidate_caches()
+        return super().train(mode)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.invalidate_caches()
+        return super()._apply(fn, *args, **kwargs)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_caches()
+        return super()._load_from_state_dict(*args, **kwargs)
+
+    def _may_keep(self, params):
+        return (not self.training) and not (torch.is_grad_enabled() and any(p.requires_grad for p in params))
+
     def _per_head(self, which):
-        """sigma (`spread`) or beta of the heads.  Where no gradient is needed the fp32 values the kernel reads are
-        kept across calls (three small launches per layer otherwise) until the parameter changes."""
+        """sigma (`spread`) or beta of the heads, as the fp32 tensor the kernel reads (kept across inference calls:
+        three small launches per layer otherwise)."""
         p = self.spread_weights if which == "spread" else self.beta_weights
         fn = self.get_spreads if which == "spread" else self.get_betas
-        if torch.is_grad_enabled() and p.requires_grad:
+        if not self._may_keep((p,)):
             return fn()
         key = (p._version, p.data_ptr(), p.dtype, self.min_spread)
         cache = self.__dict__.setdefault("_head_cache", {})
@@ -392,10 +435,9 @@ class GeoAttention(nn.Module):
         return cache[which][1]
 
     def _out_weight(self):
-        """The output projection's weight with its input columns in (heads x d_k) order.  Rebuilt whenever the
-        parameter may have changed; kept across calls only where no gradient is needed."""
+        """The output projection's weight with its input columns in (heads x d_k) order."""
         p = self.out_proj.weight
-        keep = not (torch.is_grad_enabled() and p.requires_grad)
+        keep = self._may_keep((p,))
         key = (p._version, p.data_ptr(), p.dtype)
         if keep and getattr(self, "_wo_cache", None) is not None and self._wo_cache[0] == key:
             return self._wo_cache[1]
@@ -404,10 +446,10 @@ class GeoAttention(nn.Module):
         return w_o
 
     def _fused_qkv(self):
-        """[d_model, 3*H*d_k] weight and [3*H*d_k] bias of the fused self-attention projection.  Rebuilt from the
-        per-head parameters whenever they may have changed; kept across calls only where no gradient is needed."""
+        """[d_model, 3*H*d_k] weight and [3*H*d_k] bias of the fused self-attention projection, from the per-head
+        parameters."""
         params = (self.q_proj, self.k_proj, self.v_proj, self.q_bias, self.k_bias, self.v_bias)
-        keep = not (torch.is_grad_enabled() and any(p.requires_grad for p in params))
+        keep = self._may_keep(params)
         key = tuple((p._version, p.data_ptr(), p.dtype) for p in params)
         if keep and getattr(self, "_qkv_cache", None) is not None and self._qkv_cache[0] == key:
             return self._qkv_cache[1], self._qkv_cache[2]

@@ -201,8 +201,9 @@ class _wf_embedding_learnCB(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask):
-        # the per-token partial derivatives are computed only if one of the two scales can want a gradient
-        ctx.need = bool(cb_magnitudes.requires_grad or wavenumbers.requires_grad)
+        # the per-token partial derivatives are computed only if autograd will ask for the gradient of one of the two
+        # scales (under no_grad / inference_mode it never does, whatever requires_grad says)
+        ctx.need = bool(ctx.needs_input_grad[2] or ctx.needs_input_grad[3])
         out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask, partials=ctx.need)
         if ctx.need:
             ctx.save_for_backward(d_cb, d_k)

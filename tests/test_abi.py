@@ -14,20 +14,43 @@ from proteusai_amd import _lib, synth
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(ROOT, "include", "proteus_hip.h")).read()
+def _declared(header_name):
+    header = open(os.path.join(ROOT, "include", header_name)).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = sorted(set(re.findall(r"\b(proteus_[a-z0-9_]+)\s*\(", header)))
-    assert declared, "no declarations found in the header"
+    assert declared, f"no declarations found in {header_name}"
+    return declared
+
+
+def test_library_exports_every_declared_symbol():
+    declared = _declared("proteus_hip.h")
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in proteus_hip.h but not exported"
     assert sorted(declared) == sorted(_lib.SYMBOLS)
+    # the measurement probes are not part of the product library or its header
+    assert not [n for n in declared if "probe" in n]
+    assert not hasattr(lib, "proteus_probe_valu_rate")
+
+
+def test_probe_library_exports_every_declared_symbol():
+    from proteusai_amd import _probes
+    declared = _declared("proteus_probes.h")
+    lib = ctypes.CDLL(_probes.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in proteus_probes.h but not exported"
+    assert sorted(declared) == sorted(_probes.SYMBOLS)
+    # argument errors come back before any HIP call
+    _probes.load()
+    assert _probes.load().proteus_probe_trans_valu_mix(3, 4, 256, 10, 10, None, None, None) < 0
+    assert _probes.load().proteus_probe_valu_rate(0, 1, 1, None, None) < 0
 
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.proteus_version() >= 100
+    # the binding and the header agree on the version whose argument lists they describe, and the library reports it
+    header = open(os.path.join(ROOT, "include", "proteus_hip.h")).read()
+    assert int(re.search(r"#define\s+PROTEUS_VERSION\s+(\d+)", header).group(1)) == _lib.ABI_VERSION == lib.proteus_version()
     assert lib.proteus_strerror(0) == b"ok"
     for code in range(-9, 0):
         assert lib.proteus_strerror(code) not in (b"", b"unknown error code")

@@ -55,6 +55,18 @@ def run_gpu(gpu, Q, K, V, coords, sigma, mask, tuning=0):
     return O.cpu().numpy(), L.cpu().numpy()
 
 
+
+def sample_rows(n, count, seed, tile=256):
+    """`count` distinct query rows of 0..n-1: the first and last rows, both sides of the first and last boundaries of
+    the 32-query blocks and of the 256-query workgroup tiles and of one in the middle, the rest uniformly at random."""
+    edges = {0, 1, 31, 32, 63, 64, tile - 1, tile, n // 2 - 1, n // 2, n - tile - 1, n - tile, n - 65, n - 64, n - 33, n - 32,
+             n - 2, n - 1}
+    edges = {r for r in edges if 0 <= r < n}
+    rest = np.random.default_rng(seed).permutation(n)
+    rows = list(edges) + [int(r) for r in rest if int(r) not in edges][:max(0, count - len(edges))]
+    return np.sort(np.asarray(rows, dtype=np.int32))
+
+
 def check(got, Q, K, V, coords, sigma, mask, rows=None, what=""):
     O, L = got
     Or, Lr = c_oracle.geo_attn(Q.float().numpy(), K.float().numpy(), V.float().numpy(), coords.numpy(), sigma.numpy(),
@@ -315,7 +327,9 @@ def test_cfg3_sampled_rows(gpu):
     # B=4, N=4096, H=8, d=64, Q,K,V ~ N(0,1)/8, lengths in [2048, 4096]
     Q, K, V, coords, sigma, mask = synth.attn_inputs(4, 8, 4096, 64, seed=3, min_len=2048)
     got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
-    rows = np.sort(np.random.default_rng(3).choice(4096, 64, replace=False)).astype(np.int32)
+    # 160 query rows x 8 heads x 4 batch items (padded rows among them: they must be exact zeros), ends of the sequence,
+    # of the 32-query blocks and of the 256-query tiles included
+    rows = sample_rows(4096, 160, seed=3)
     check(got, Q, K, V, coords, sigma, mask, rows=rows, what="cfg3")
 
 
@@ -332,7 +346,7 @@ def test_cfg5_sampled_rows(gpu):
     wc, _ = synth.we_inputs(65536, seed=5, compact=True)
     Q, K, V, coords, sigma, mask = synth.attn_inputs(1, 8, 16384, 64, seed=5, coords=wc[:, :16384].contiguous())
     got = run_gpu(gpu, Q, K, V, coords, sigma, mask)
-    rows = np.sort(np.random.default_rng(5).choice(16384, 32, replace=False)).astype(np.int32)
+    rows = sample_rows(16384, 160, seed=5)              # 160 query rows x 8 heads, tile boundaries and both ends included
     check(got, Q, K, V, coords, sigma, mask, rows=rows, what="cfg5")
     # size-independent property at full size: V = 1 -> O = 1
     O1, _ = run_gpu(gpu, Q, K, torch.ones_like(V), coords, sigma, None)

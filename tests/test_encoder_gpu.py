@@ -93,12 +93,35 @@ def test_cfg4_shape_inference_path_equals_the_path_autograd_records(gpu):
                 layer.attn.spread_weights.add_(0.5)
             moved = model(coords, tokens, mask).float().cpu()
         assert not torch.equal(fast[valid], moved[valid])
+        # a write through `.data` (how EMA weights are swapped in) bumps no version counter: in eval() mode the kept
+        # constants are dropped by invalidate_caches() or another eval() call, and then the result follows
+        with torch.no_grad():
+            for layer in model.layers:
+                layer.attn.out_proj.weight.data.mul_(1.5)
+                layer.attn.q_proj.data.mul_(0.5)
+                layer.attn.invalidate_caches()
+            swapped = model(coords, tokens, mask).float().cpu()
+            for layer in model.layers:
+                layer.attn.spread_weights.data.add_(0.5)
+            model.eval()
+            swapped2 = model(coords, tokens, mask).float().cpu()
+        assert not torch.equal(moved[valid], swapped[valid]) and not torch.equal(swapped[valid], swapped2[valid])
+        # in training mode nothing is kept: a `.data` write shows at once, also under no_grad
+        model.train()
+        with torch.no_grad():
+            t1 = model(coords, tokens, mask).float().cpu()
+            for layer in model.layers:
+                layer.attn.out_proj.weight.data.mul_(1.25)
+            t2 = model(coords, tokens, mask).float().cpu()
+        assert not torch.equal(t1[valid], t2[valid])
 
 
 def test_cfg4_shape_embedding_and_first_attention_on_sampled_rows(gpu):
-    """At the real shape (B=8, N=1024, d_model=512, H=8, bf16 weights, fp32 WE, lengths in [128, 1024]) a dense oracle of
-    the whole stack takes too long for a test, but rows are independent in both kernels: the embedding and the first
-    layer's attention (fed with the activations the model itself produces) are checked on sampled rows."""
+    """At the real shape (B=8, N=1024, d_model=512, H=8, bf16 weights, fp32 WE, lengths in [128, 1024]) the two kernels
+    in isolation, held to their own bars: rows are independent in both, so the embedding and the first layer's
+    attention (fed with the activations the model itself produces) are checked on sampled rows against the C oracles.
+    (The logits of the whole stack are compared with the CPU statement of the stack in
+    test_cfg4_shape_logits_match_the_cpu_statement_of_the_whole_stack.)"""
     torch.manual_seed(4)
     model = pa.ProteusEncoder().eval().to(gpu)
     model.aa_embedding.to(torch.bfloat16)
@@ -139,6 +162,55 @@ def test_cfg4_shape_embedding_and_first_attention_on_sampled_rows(gpu):
         assert np.abs(O - Or).max() <= 2e-2 * vmax / 4, f"first-layer attention at the encoder's shape: {np.abs(O - Or).max():.3e} (max |V| {vmax:.2f})"
         assert np.abs(L[fin] - Lr[fin]).max() <= 4e-3
         assert (O[~fin] == 0).all()
+
+
+def _cfg4_batch():
+    g = torch.Generator().manual_seed(4)
+    coords = torch.stack([synth.random_walk_chain(1024, g) for _ in range(8)])
+    tokens = torch.randint(0, 33, (8, 1024), generator=g)
+    lens = torch.randint(128, 1025, (8,), generator=g)
+    mask = torch.arange(1024)[None, :] >= lens[:, None]
+    return coords, tokens, mask
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32_weights", "bf16_weights"])
+def test_cfg4_shape_logits_match_the_cpu_statement_of_the_whole_stack(gpu, dtype):
+    """The whole encoder at BASELINE.json configs[3] (B=8, N=1024, d_model=512, H=8, 4 layers, FFN 2048, head to 20
+    logits, lengths in [128, 1024]) against the fp32 CPU statement of the same stack with the same weights
+    (torch_oracle.encoder_forward_torch: dense torch attention and embedding oracles, pinned in
+    tests/test_oracle_encoder.py), on every valid token.
+
+    Bars.  fp32 weights: the only low-precision steps are the attention's bf16 operands and probabilities (four
+    layers): rel-L2 over all valid logits <= 5e-3, max-abs <= 1 % of the logits' range.  bf16 weights (the
+    configuration BASELINE names): every activation between two layers is rounded to bf16 (2^-9 relative, some 30
+    roundings from the embedding to the head, which LayerNorm renormalises rather than damps): rel-L2 <= 2e-2, per
+    token rel-L2 <= 8e-2 on every token, max-abs <= 4 % of the logits' range, and the arg-max amino acid agrees where
+    the reference's top two logits are further apart than that."""
+    torch.manual_seed(4)
+    model = pa.ProteusEncoder().eval().to(gpu)
+    model.aa_embedding.to(dtype)
+    model.layers.to(dtype)
+    model.head.to(dtype)
+    coords, tokens, mask = _cfg4_batch()
+    with torch.no_grad():
+        out = model(coords.to(gpu), tokens.to(gpu), mask.to(gpu)).float().cpu()
+    ref = torch_oracle.encoder_forward_torch(model.state_dict(), model.layers[0].attn.min_spread, coords, tokens, mask)
+    valid = ~mask
+    got, want = out[valid].double(), ref[valid].double()
+    assert got.shape == want.shape and got.shape[1] == 20 and torch.isfinite(got).all()
+    rel = float((got - want).norm() / want.norm())
+    per_token = ((got - want).norm(dim=1) / want.norm(dim=1))
+    span = float(want.max() - want.min())
+    max_abs = float((got - want).abs().max())
+    print(f"encoder at configs[3], {dtype}: rel-L2 {rel:.3e}, worst token {float(per_token.max()):.3e}, "
+          f"max abs {max_abs:.3e} of a logit range of {span:.2f}", flush=True)
+    bars = {torch.float32: (5e-3, 3e-2, 0.01), torch.bfloat16: (2e-2, 8e-2, 0.04)}[dtype]
+    assert rel <= bars[0], f"rel-L2 {rel:.3e}"
+    assert float(per_token.max()) <= bars[1], f"worst token rel-L2 {float(per_token.max()):.3e}"
+    assert max_abs <= bars[2] * span, f"max abs {max_abs:.3e}, range {span:.2f}"
+    top2 = want.topk(2, dim=1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2 * bars[2] * span
+    assert clear.sum() > 0 and torch.equal(got.argmax(dim=1)[clear], want.argmax(dim=1)[clear])
 
 
 def test_forward_replays_bit_equal_from_a_captured_graph(gpu):

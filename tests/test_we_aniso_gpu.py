@@ -179,6 +179,27 @@ def test_embedding_alone_equals_the_embedding_with_partials(gpu, tuning):
     with torch.no_grad():
         y = pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu)).cpu().numpy()
     assert rel_l2(y, full) <= 1e-6
+    # learnable scales under no_grad / inference_mode: no gradient will be asked for, so the partial derivatives are not
+    # produced either (the forward is called with partials=False)
+    import proteusai_amd.wf_embedding as wfe
+    seen = []
+    real = wfe.we_aniso_forward
+
+    def spy(*args, **kwargs):
+        seen.append(kwargs.get("partials"))
+        return real(*args, **kwargs)
+    wfe.we_aniso_forward = spy
+    try:
+        cbg, wng = cb.to(gpu).requires_grad_(True), wn.to(gpu).requires_grad_(True)
+        with torch.no_grad():
+            y2 = pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), cbg, wng, mask.to(gpu))
+        with torch.inference_mode():
+            pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), cbg, wng, mask.to(gpu))
+        y3 = pa.wf_embedding_learnCB(a.to(gpu), b.to(gpu), cbg, wng, mask.to(gpu))
+    finally:
+        wfe.we_aniso_forward = real
+    assert seen == [False, False, True] and not y2.requires_grad and y3.requires_grad
+    assert rel_l2(y2.cpu().numpy(), full) <= 1e-6
     c = a.to(gpu).requires_grad_(True)                    # some other input wants a gradient: backward returns none for all
     pa.wf_embedding_learnCB(c, b.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu)).sum().backward()
     assert c.grad is None

@@ -62,3 +62,35 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(gpu):
     assert lib.proteus_we_bwd_static(p, p, p, p, 0, 8, 4, None) == -2
     assert lib.proteus_we_bwd_static(p + 4, p, p, p, 1, 8, 4, None) == -5
     assert b"capacity" in lib.proteus_strerror(-8)
+
+
+def test_static_scratch_entry_point_replays_from_a_captured_graph(gpu):
+    """The use the entry point exists for.  The first call per GPU resolves the scratch array's address and is made
+    eagerly (the tests above did, and so does the warm-up here); after that a call only launches its two kernels and
+    can be captured.  Replays, with eager calls on other inputs between them, reproduce the eager result to the bit."""
+    lib = _lib.load()
+    Z, N, K = 2, 3000, 256
+    dO, c, s = _inputs(gpu, Z, N, K, 11)
+    other = _inputs(gpu, 1, 500, 512, 12)
+    out = torch.full((K,), float("nan"), dtype=torch.float32, device=gpu)
+    eager = _static(lib, dO, c, s, Z, N, K, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _static(lib, dO, c, s, Z, N, K, ctypes.c_void_p(side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.proteus_we_bwd_static(dO.data_ptr(), c.data_ptr(), s.data_ptr(), out.data_ptr(), Z, N, K,
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.proteus_strerror(rc)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        out.fill_(float("nan"))
+        _static(lib, *other, 1, 500, 512, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))   # dirties the shared array
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
