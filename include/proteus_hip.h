@@ -260,6 +260,35 @@ int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint1
                                int Z, int H, int N, int d_head, int tuning);
 
 /*
+ * proteus_geo_attn_fwd with a caller-provided workspace, for batches that come with a padding mask (d_head = 64).
+ * The reference's launch gives every (batch, head, query tile) one program whose key loop is as long as the sequence
+ * (old/old_scripts/attn/geometric_attn.py:586-599), so a padded batch lasts as long as its longest sequence.  With a
+ * workspace the work is cut into equal shares instead (key tiles of one item may go to several workgroups, whose
+ * partial results meet in the workspace).  Same result as proteus_geo_attn_fwd to fp32 rounding of the final
+ * normalisation (the partial sums of a query are added in a different order).
+ *   strides      as proteus_geo_attn_fwd_strided, or NULL for contiguous [Z,H,N,d_head] tensors
+ *   workspace    device memory, 256-byte aligned, workspace_bytes >= proteus_geo_attn_fwd_workspace_bytes(Z, H, N,
+ *                d_head, tuning); not initialised by the caller, nothing kept in it between calls; calls that share
+ *                one workspace must not overlap.  NULL / too small (or a shape for which
+ *                proteus_geo_attn_fwd_workspace_bytes returns 0, or key_pad_mask == NULL): the call is
+ *                proteus_geo_attn_fwd[_strided].
+ *   tuning       0 = automatic: the balanced schedule for N > 1024 and at least 24576 (item, key tile) steps of the full batch;
+ *                8 = the balanced schedule wherever it is possible (d_head = 64, Z <= 256, fewer than 2^30 steps);
+ *                proteus_geo_attn_fwd_workspace_bytes returns 0 where the given tuning does not take it
+ * Launches (balanced path): a plan kernel, the persistent grid, and the plain grid, which returns at once unless a
+ * query tile's tokens lie too far apart for the matrix-core distances (then it does the whole batch instead).
+ */
+size_t proteus_geo_attn_fwd_workspace_bytes(int Z, int H, int N, int d_head, int tuning);
+int proteus_geo_attn_fwd_ws(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,
+                            const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                            float* O, float* L, void* workspace, size_t workspace_bytes,
+                            int Z, int H, int N, int d_head, int tuning, void* stream);
+int proteus_geo_attn_fwd_ws_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,
+                                  const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                  const float* O, const float* L, const void* workspace, size_t workspace_bytes,
+                                  int Z, int H, int N, int d_head, int tuning);
+
+/*
  * The same kernel with the logits of the reference's Triton kernel instead of
  * the README multiplier (old/old_scripts/attn/geometric_attn.py:193-201, launch
  * :588-599; dense statement tests/attn/geo_attn.py:194-210):

@@ -22,6 +22,7 @@ SYMBOLS = [
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
     "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_bwd_static", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
+    "proteus_geo_attn_fwd_workspace_bytes", "proteus_geo_attn_fwd_ws", "proteus_geo_attn_fwd_ws_check",
     "proteus_geo_attn_bwd_check", "proteus_geo_attn_fwd_strided", "proteus_geo_attn_fwd_strided_check",
     "proteus_geo_attn_legacy_fwd_strided",
     "proteus_geo_attn_bwd_strided", "proteus_geo_attn_bwd_strided_check", "proteus_geo_attn_num_variants",
@@ -104,6 +105,12 @@ def load():
     lib.proteus_geo_attn_bwd_strided.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, ci, vp]
     lib.proteus_geo_attn_bwd_strided_check.restype = ci
     lib.proteus_geo_attn_bwd_strided_check.argtypes = [vp] * 4 + [i64p] + [vp] * 11 + [ci, ci, ci, ci, cf, cf, ci]
+    lib.proteus_geo_attn_fwd_workspace_bytes.restype = sz
+    lib.proteus_geo_attn_fwd_workspace_bytes.argtypes = [ci, ci, ci, ci, ci]
+    lib.proteus_geo_attn_fwd_ws.restype = ci
+    lib.proteus_geo_attn_fwd_ws.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, vp, sz, ci, ci, ci, ci, ci, vp]
+    lib.proteus_geo_attn_fwd_ws_check.restype = ci
+    lib.proteus_geo_attn_fwd_ws_check.argtypes = [vp, vp, vp, i64p, vp, vp, vp, vp, vp, vp, sz, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_fwd_check.restype = ci
     lib.proteus_geo_attn_fwd_check.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     lib.proteus_geo_attn_num_variants.restype = ci

@@ -55,21 +55,41 @@ namespace {
 #include "geo_attn_fwd_body.inc"
 #include "geo_attn_fwd_pipe.inc"
 
+// True if the plan of a padded batch (see geo_attn_plan_kernel) marks a query tile whose tokens spread too far for
+// the matrix-core distances: then the balanced kernel leaves the launch to the plain grid.
+// (`any_wide`: an int of the workgroup's LDS, free at that point)
+__device__ __forceinline__ bool ga_plan_has_wide_tile(const int* __restrict__ wide, const int n, int& any_wide) {
+    if (threadIdx.x == 0) any_wide = 0;
+    __syncthreads();
+    int w = 0;
+    for (int i = threadIdx.x; i < n; i += GA_THREADS) w |= wide[i];
+    if (w) any_wide = 1;
+    __syncthreads();
+    const bool r = any_wide != 0;
+    __syncthreads();
+    return r;
+}
+
 // The pipelined body over the first half of a doubled grid, the direct-distance body (for workgroups whose
 // queries are spread too widely for the matrix-core distances) over the second; take_all: the pipelined body alone.
+// gate != NULL: the launch follows a balanced one over the same batch and does the work only if that one declined
+// (a query tile too wide for the matrix-core distances: gate[0 .. gate_n) holds a non-zero flag).
 __global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                               const uint16_t* __restrict__ V, const float* __restrict__ coords,
                               const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                               float* __restrict__ O, float* __restrict__ L,
                               const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs, const int take_all,
+                              const int* __restrict__ gate, const int gate_n, const int num_cus,
                               const GaStrides st)
 {
     extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
+    if (gate && !ga_plan_has_wide_tile(gate, gate_n, reinterpret_cast<PipeSmem*>(ga_dyn_smem)->n_eff)) return;
     const int id = (int)blockIdx.x;
     if (id < n_wgs)
+        // (workgroups are handed to the compute units in turn: num_cus apart they share one)
         geo_attn_fwd_pipe_body(*reinterpret_cast<PipeSmem*>(ga_dyn_smem), id, Q, K, V, coords, sigma, key_pad, O, L,
-                               H, N, ZH, n_qtiles, take_all, st);
+                               H, N, ZH, n_qtiles, take_all, (id / num_cus) & 1, st);
     else
         geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), id - n_wgs, Q, K, V, coords, sigma, key_pad, O, L,
                                           H, N, ZH, n_qtiles, 0, nullptr, 0.f, 1.f, st);
@@ -77,9 +97,235 @@ void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __
 constexpr size_t GA_PIPE_LDS = sizeof(PipeSmem) > sizeof(Smem) ? sizeof(PipeSmem) : sizeof(Smem);
 static_assert(GA_PIPE_LDS <= 80 * 1024, "two workgroups per compute unit");
 
+// ---------------- padded batches: a balanced schedule over a persistent grid ----------------
+//
+// With a padding mask the plain grid gives every (batch, head, 256-query tile) one workgroup, whose key loop is as
+// long as its sequence: when the grid is about one round of the chip, the launch lasts as long as the longest
+// sequence's workgroups while the others' slots idle.  Here the work is laid out as one line of steps (a step = one
+// key tile of one item; items ordered batch, head, query tile; only query tiles and key tiles up to the last unpadded
+// token count) and cut into G equal shares, one per persistent workgroup.  A share is a few parts: the tail of one
+// item, whole items, the head of another.  Every part leaves its unnormalised state in the caller's workspace; the
+// last of an item's parts to finish (a counter per item says which) adds them up and writes O and L.  No workgroup
+// ever waits for another.  The plan that all workgroups derive the same shares from (last unpadded token per query
+// tile) is made by a small kernel launched before this one.
+
+constexpr int    GB_MAX_WGS     = 512;                       // persistent workgroups: two per compute unit of a 256-CU chip
+constexpr int    GB_MAX_Z       = 256;                       // batch items (their lengths and prefix sums live in LDS)
+constexpr size_t GB_PART_FLOATS = (size_t)GP_PART_FLOATS;   // one part: the O^T accumulators of 256 queries, (reference, row sum) per query
+
+struct BalSmem {
+    PipeSmem pipe;
+    int n_eff[GB_MAX_Z];             // 1 + index of the last unpadded token of a batch item
+    int prefix[GB_MAX_Z + 1];        // steps before batch item z
+    int flag;
+};
+static_assert(sizeof(BalSmem) <= 80 * 1024, "two workgroups per compute unit");
+
+// Ints of the plan at the head of the workspace: tile_last [Z * nqt], wide [Z * nqt], counters [Z * nqt * H].
+__host__ __device__ inline size_t gb_plan_ints(const int Z, const int H, const int nqt) { return (size_t)Z * nqt * (2 + (size_t)H); }
+__host__ __device__ inline size_t gb_parts_offset(const int Z, const int H, const int nqt) {
+    return (gb_plan_ints(Z, H, nqt) * sizeof(int) + 255) / 256 * 256;
+}
+
+// One workgroup per (query tile, batch item): 1 + index of its last unpadded token, whether its unpadded tokens lie
+// too far apart for the matrix-core distances of the pipelined body at the smallest sigma (same origin as the body:
+// midway between the first and the last unpadded token of the tile), and zeroed part counters of its H items.
+__global__ __launch_bounds__(GA_THREADS)
+void geo_attn_plan_kernel(const float* __restrict__ coords, const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                          int* __restrict__ plan, const int Z, const int H, const int N, const int nqt)
+{
+    __shared__ int s_lo, s_hi;
+    __shared__ unsigned s_rho2;
+    const int qt = (int)blockIdx.x, z = (int)blockIdx.y, tid = (int)threadIdx.x;
+    int* tile_last = plan;
+    int* wide      = plan + (size_t)Z * nqt;
+    int* counters  = plan + (size_t)2 * Z * nqt;
+    if (tid == 0) { s_lo = 0x7fffffff; s_hi = -1; s_rho2 = 0u; }
+    __syncthreads();
+    const int q = qt * GA_THREADS + tid;
+    const bool valid = q < N && !(key_pad && key_pad[(size_t)z * N + q]);
+    const float* cz = coords + (size_t)z * N * 3;
+    float cx = 0.f, cy = 0.f, cw = 0.f;
+    if (valid) { cx = cz[3 * q]; cy = cz[3 * q + 1]; cw = cz[3 * q + 2]; }
+    {
+        // first and last unpadded token of the wave from one ballot; one LDS atomic per wave
+        const uint64_t bal = __builtin_amdgcn_ballot_w64(valid);
+        if ((tid & 63) == 0 && bal != 0) {
+            const int base = qt * GA_THREADS + (tid & ~63);
+            atomicMin(&s_lo, base + __builtin_ctzll(bal));
+            atomicMax(&s_hi, base + 63 - __builtin_clzll(bal));
+        }
+    }
+    __syncthreads();
+    const int lo = s_lo, hi = s_hi;
+    if (hi >= 0) {
+        const float ox = 0.5f * (cz[3 * lo] + cz[3 * hi]), oy = 0.5f * (cz[3 * lo + 1] + cz[3 * hi + 1]), oz = 0.5f * (cz[3 * lo + 2] + cz[3 * hi + 2]);
+        const float dx = cx - ox, dy = cy - oy, dz = cw - oz;
+        float r2 = valid ? dx * dx + dy * dy + dz * dz : 0.f;
+        for (int o = 32; o > 0; o >>= 1) r2 = fmaxf(r2, __shfl_xor(r2, o));
+        if ((tid & 63) == 0) atomicMax(&s_rho2, __builtin_bit_cast(unsigned, r2));
+    }
+    __syncthreads();
+    const size_t t = (size_t)z * nqt + qt;
+    if (tid == 0) {
+        float cs_max = 0.f;
+        for (int h = 0; h < H; ++h) cs_max = fmaxf(cs_max, 0.84932180028801907f / sigma[h]);
+        tile_last[t] = hi + 1;
+        // (a sigma that is not a positive number gives garbage either way; NaN compares false: the plain grid's
+        // behaviour is kept by calling the tile wide)
+        const float rho2 = __builtin_bit_cast(float, s_rho2) * cs_max * cs_max;
+        wide[t] = (hi >= 0 && !(rho2 <= GA_MFMA_DIST_MAX_RHO2)) ? 1 : 0;
+    }
+    for (int h = tid; h < H; h += GA_THREADS) counters[t * H + h] = 0;
+}
+
+__global__ __launch_bounds__(GA_THREADS, 2)
+void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                                  const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                                  const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                                  float* __restrict__ O, float* __restrict__ L,
+                                  int* __restrict__ plan, float* __restrict__ parts,
+                                  const int Z, const int H, const int N, const int nqt, const GaStrides st)
+{
+    extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
+    BalSmem& bs = *reinterpret_cast<BalSmem*>(ga_dyn_smem);
+    const int tid = (int)threadIdx.x;
+    const int G = (int)gridDim.x;
+    const int* tile_last = plan;
+    const int* wide      = plan + (size_t)Z * nqt;
+    int*       counters  = plan + (size_t)2 * Z * nqt;
+
+    // ---- the plan every workgroup derives: lengths, steps before each batch item ----
+    if (ga_plan_has_wide_tile(wide, Z * nqt, bs.flag)) return; // the plain grid, launched next, does this batch
+    for (int z = tid; z < Z; z += GA_THREADS) {
+        int last = 0;
+        for (int qt = 0; qt < nqt; ++qt) last = max(last, tile_last[(size_t)z * nqt + qt]);
+        bs.n_eff[z] = last;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int z = 0; z < Z; ++z) {
+            bs.prefix[z] = run;
+            const int ne = bs.n_eff[z];
+            run += H * ((ne + GA_THREADS - 1) / GA_THREADS) * ((ne + GA_BN - 1) / GA_BN);
+        }
+        bs.prefix[Z] = run;
+    }
+    __syncthreads();
+    const int total = bs.prefix[Z];
+    const int share = max((total + G - 1) / G, 1);
+    // consecutive workgroup numbers go to different XCDs: XCD x takes the x-th eighth of the line, so that the
+    // workgroups that share an L2 work on neighbouring items (the same K and V)
+    const int g = ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3);
+
+    int a = min(g * share, total);
+    const int b = min(a + share, total);
+    while (a < b) {
+        int z = 0;
+        while (bs.prefix[z + 1] <= a) ++z;                      // (uniform: a few scalar steps)
+        z = __builtin_amdgcn_readfirstlane(z);
+        const int ne = bs.n_eff[z];
+        const int nq = (ne + GA_THREADS - 1) / GA_THREADS, c = (ne + GA_BN - 1) / GA_BN;
+        const int r = a - bs.prefix[z];
+        const int item = r / c, k0 = r - item * c;
+        const int h = item / nq, qt = item - h * nq;
+        const int zh = z * H + h;
+        const int start = a - k0;                               // first step of the item on the line
+        const int k1 = min(c, k0 + (b - a));
+        // the workgroups that hold parts of this item, and where each left (or will leave) its part: a workgroup's
+        // slot 0 takes the item its share begins with, slot 1 an item that begins inside its share and ends beyond it
+        const int first_g = start / share, last_g = (start + c - 1) / share;
+        const int nparts = last_g - first_g + 1;
+        auto slot_of = [&](const int j) -> float* {
+            const int second = (j == first_g && start > j * share) ? 1 : 0;
+            return parts + ((size_t)2 * j + second) * GB_PART_FLOATS;
+        };
+        float* mine = slot_of(g);
+        const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, mine, (2 * (int)blockIdx.x >= G) ? 1 : 0,
+                                                    Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
+        if (rc == 0) {
+            // The part was written with device-scope stores: once they have completed it is in memory for every
+            // workgroup of the chip, and only then may the item's counter say so.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) bs.flag = (nparts == 1) ? 1 : (atomicAdd(&counters[((size_t)z * nqt + qt) * H + h], 1) == nparts - 1);
+            __syncthreads();
+            if (bs.flag) {
+                // the last part of the item to finish adds them up, in the registers' layout: with M the largest
+                // reference among the parts that saw a key, O = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p.
+                // (The loads of a part are issued together: one round trip to memory per part and pass.)
+                const int wave = tid >> 6, lane = tid & 63, half = lane >> 5, col = lane & 31;
+                float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
+                const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
+#pragma unroll 1
+                for (int bq = 0; bq < 2; ++bq) {
+                    const int mlo = gp_part_ml_offset(wave, bq, col);
+                    float M = -INFINITY;
+                    for (int j = first_g; j <= last_g; ++j) {
+                        const floatx2 ml = __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(gp_part_rsrc(slot_of(j)), mlo, 0, GP_SC1));
+                        if (ml[1] > 0.f) M = fmaxf(M, ml[0]);
+                    }
+                    float l = 0.f;
+                    float acc[32];
+#pragma unroll
+                    for (int r = 0; r < 32; ++r) acc[r] = 0.f;
+                    for (int j = first_g; j <= last_g; ++j) {
+                        const __amdgpu_buffer_rsrc_t rp = gp_part_rsrc(slot_of(j));
+                        const gp_uint2v rml = __builtin_amdgcn_raw_buffer_load_b64(rp, mlo, 0, GP_SC1);
+                        uint4v raw[8];
+#pragma unroll
+                        for (int q4 = 0; q4 < 8; ++q4)
+                            raw[q4] = __builtin_amdgcn_raw_buffer_load_b128(rp, gp_part_o_offset(wave, bq, q4 >> 2, q4 & 3, lane), 0, GP_SC1);
+                        const floatx2 ml = __builtin_bit_cast(floatx2, rml);
+                        const float w = (ml[1] > 0.f) ? __builtin_amdgcn_exp2f(ml[0] - M) : 0.f;
+                        l = __builtin_fmaf(w, ml[1], l);
+#pragma unroll
+                        for (int q4 = 0; q4 < 8; ++q4) {
+                            const floatx4 v = __builtin_bit_cast(floatx4, raw[q4]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(w, v[e], acc[4 * q4 + e]);
+                        }
+                    }
+                    const int qi = qt * (GA_WAVES * 64) + wave * 64 + 32 * bq + col;
+                    if (qi < N) {
+                        const bool row_ok = l > 0.f && !(mz && mz[qi]);
+                        const float inv_l = row_ok ? 1.0f / l : 0.f;
+                        float* orow = Oh + (size_t)qi * (size_t)st.o[2];
+#pragma unroll
+                        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                            for (int gq = 0; gq < 4; ++gq)
+                                *reinterpret_cast<float4*>(orow + dt * 32 + 8 * gq + 4 * half) =
+                                    make_float4(acc[dt * 16 + 4 * gq] * inv_l, acc[dt * 16 + 4 * gq + 1] * inv_l,
+                                                acc[dt * 16 + 4 * gq + 2] * inv_l, acc[dt * 16 + 4 * gq + 3] * inv_l);
+                        if (L && half == 0) L[(size_t)zh * N + qi] = row_ok ? (M + __log2f(l)) * 0.69314718055994531f : -INFINITY;
+                    }
+                }
+            }
+        }
+        a += k1 - k0;
+    }
+
+    // ---- query tiles behind the last unpadded token of their sequence: zeros, L = -inf ----
+    for (int e = (int)blockIdx.x; e < Z * H * nqt; e += G) {
+        const int z = e / (H * nqt), rem = e - z * (H * nqt);
+        const int h = rem / nqt, qt = rem - h * nqt;
+        if (qt * GA_THREADS < bs.n_eff[z]) continue;
+        float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
+        const int chunk = tid & 15;
+        for (int ql = tid >> 4; ql < GA_THREADS; ql += GA_THREADS / 16) {
+            const int qi = qt * GA_THREADS + ql;
+            if (qi >= N) break;
+            *reinterpret_cast<float4*>(Oh + (size_t)qi * (size_t)st.o[2] + 4 * chunk) = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (L && chunk == 0) L[((size_t)z * H + h) * N + qi] = -INFINITY;
+        }
+    }
+}
+
 struct GaVariant { const char* name; };
 const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"},
-                                {"pipelined"}, {"pipelined_dist_mfma"}, {"split_keys"} };
+                                {"pipelined"}, {"pipelined_dist_mfma"}, {"split_keys"}, {"balanced"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -107,42 +353,123 @@ extern "C" int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, 
 }
 
 namespace {
-int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
-                     const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, bool take_all,
-                     const GaStrides& gs, hipStream_t st)
-{
-    // more than 64 KB of dynamic LDS must be allowed once per device (remembered for the first 64 devices)
-    static std::atomic<unsigned long long> allowed{0ull};
+// more than 64 KB of dynamic LDS must be allowed once per kernel and device (remembered for the first 64 devices)
+int allow_lds(const void* kernel, size_t bytes, std::atomic<unsigned long long>& allowed) {
     int dev = 0;
     const hipError_t got = hipGetDevice(&dev);
     if (got != hipSuccess) return (int)got;
     if (dev < 0 || dev >= 64 || !((allowed.load(std::memory_order_relaxed) >> dev) & 1ull)) {
-        const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)GA_PIPE_LDS);
+        const hipError_t attr = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (attr != hipSuccess) return (int)attr;
         if (dev >= 0 && dev < 64) allowed.fetch_or(1ull << dev, std::memory_order_relaxed);
     }
+    return (int)hipSuccess;
+}
+
+// Compute units of the current device, looked up once per device.
+int device_cus(int* cus_out) {
+    static std::atomic<int> cached[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    int cus = (dev >= 0 && dev < 64) ? cached[dev].load(std::memory_order_relaxed) : 0;
+    if (cus == 0) {
+        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return (int)e;
+        if (cus < 1) cus = 1;
+        if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    *cus_out = cus;
+    return (int)hipSuccess;
+}
+
+int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                     const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, bool take_all,
+                     const int* gate, int gate_n, const GaStrides& gs, hipStream_t st)
+{
+    static std::atomic<unsigned long long> allowed{0ull};
+    const int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel), GA_PIPE_LDS, allowed);
+    if (rc != (int)hipSuccess) return rc;
     constexpr int BM = GA_WAVES * 64;
     const int n_qtiles = (N + BM - 1) / BM;
     const int ZH = Z * H;
     const unsigned n_wgs = (unsigned)n_qtiles * (unsigned)ZH;
+    int cus = 0;
+    const int rc2 = device_cus(&cus);
+    if (rc2 != (int)hipSuccess) return rc2;
     hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
-                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gs);
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gate, gate_n, cus, gs);
     return (int)hipGetLastError();
+}
+
+// Number of persistent workgroups of the balanced launch on the current device: two per compute unit, a multiple of 8
+// (one eighth of the line of steps per XCD), at most GB_MAX_WGS.
+int balanced_grid(int* G) {
+    int cus = 0;
+    const int rc = device_cus(&cus);
+    if (rc != (int)hipSuccess) return rc;
+    int g = 2 * cus;
+    if (g > GB_MAX_WGS) g = GB_MAX_WGS;
+    g &= ~7;
+    if (g < 8) g = 8;
+    *G = g;
+    return (int)hipSuccess;
+}
+
+// Is the balanced schedule possible for this shape (a padding mask, the pipelined body's head dimension, lengths and
+// prefix sums that fit the workgroup's LDS and 31-bit arithmetic) and, unless `forced`, worth taking: sequences long
+// enough that a workgroup's share holds a few parts at most and each part many key tiles.  From the shape alone.
+bool balanced_applies(const uint8_t* key_pad_mask, int Z, int H, int N, int d_head, bool forced) {
+    if (!key_pad_mask || d_head != GA_D || Z > GB_MAX_Z) return false;
+    const long nqt = (N + GA_THREADS - 1) / GA_THREADS, c = (N + GA_BN - 1) / GA_BN;
+    const long steps = (long)Z * H * nqt * c;
+    if (steps >= (1L << 30)) return false;
+    // (measured: 4 x 8 x 4096 with lengths 2344-3702 168 -> 151 us, 2 x 8 x 8192 160 -> 136 us; 8 x 8 x 2048 with 32 steps per
+    // workgroup on a full batch 111 -> 128 us: every part of an item costs a prologue of about four key tiles' time)
+    return forced || (N > 1024 && steps >= 48L * GB_MAX_WGS);
+}
+
+// Plan, balanced launch, and the plain grid gated on the plan (it runs only if the balanced launch declined).
+int launch_attn_balanced(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                         const uint8_t* key_pad_mask, float* O, float* L, void* workspace, int Z, int H, int N,
+                         const GaStrides& gs, hipStream_t st)
+{
+    static std::atomic<unsigned long long> allowed{0ull};
+    int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_balanced_kernel), sizeof(BalSmem), allowed);
+    if (rc != (int)hipSuccess) return rc;
+    int G = 0;
+    rc = balanced_grid(&G);
+    if (rc != (int)hipSuccess) return rc;
+    const int nqt = (N + GA_THREADS - 1) / GA_THREADS;
+    int*   plan  = static_cast<int*>(workspace);
+    float* parts = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gb_parts_offset(Z, H, nqt));
+    hipLaunchKernelGGL(geo_attn_plan_kernel, dim3(nqt, Z), dim3(GA_THREADS), 0, st, coords, sigma, key_pad_mask, plan, Z, H, N, nqt);
+    hipLaunchKernelGGL(geo_attn_fwd_balanced_kernel, dim3(G), dim3(GA_THREADS), sizeof(BalSmem), st,
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, plan, parts, Z, H, N, nqt, gs);
+    rc = (int)hipGetLastError();
+    if (rc != (int)hipSuccess) return rc;
+    return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, false, plan + (size_t)Z * nqt, Z * nqt, gs, st);
 }
 
 // d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
 // the software-pipelined kernel runs (automatically for large grids of long sequences, or when the tuning asks).
 int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords,
                 const float* sigma, const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
-                const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
+                const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st,
+                void* workspace = nullptr, size_t workspace_bytes = 0)
 {
+    const bool pipe_tuning = tuning == 5 || tuning == 6 || tuning == 8;
     if (d_head == 32)
-        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 0 : tuning,
+        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,
                                               beta, min_rbf, max_rbf, gs, st);
     if (d_head == 128)
-        return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 0 : tuning,
+        return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,
                                                beta, min_rbf, max_rbf, gs, st);
+    // A padded batch of long sequences, with a workspace to exchange partial results in: the balanced schedule.
+    if (!legacy && (tuning == 0 || tuning == 8) && workspace && balanced_applies(key_pad_mask, Z, H, N, d_head, tuning == 8)
+        && workspace_bytes >= proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d_head, tuning))
+        return launch_attn_balanced(Q, K, V, coords, sigma, key_pad_mask, O, L, workspace, Z, H, N, gs, st);
+    if (tuning == 8) tuning = 0;
     // The pipelined kernel pays a longer prologue back from about 16 key tiles per workgroup on, and only where its
     // 256-query workgroups fill the chip twice: measured against the templated body it wins from 512 workgroups and
     // N = 1024 on (3-11 %), loses below (7-9 % at 256 workgroups of N = 1024, 6-10 % at N = 256 and 512).  A batch that
@@ -151,7 +478,7 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
     const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
     if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
-        return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
+        return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, nullptr, 0, gs, st);
     return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
 }
@@ -219,6 +546,49 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
     if (rc != PROTEUS_OK) return rc;
     return launch_attn(false, false, d_head, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f,
                        contiguous_strides(H, N, d_head), reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t proteus_geo_attn_fwd_workspace_bytes(int Z, int H, int N, int d_head, int tuning)
+{
+    if (Z <= 0 || H <= 0 || N <= 0 || N > PROTEUS_ATTN_MAX_N || (long)Z * H > 65535) return 0;
+    if (tuning != 0 && tuning != 8) return 0;
+    // (whether a mask will be passed is not known here: sized as if)
+    if (!balanced_applies(reinterpret_cast<const uint8_t*>(1), Z, H, N, d_head, tuning == 8)) return 0;
+    const int nqt = (N + GA_THREADS - 1) / GA_THREADS;
+    return gb_parts_offset(Z, H, nqt) + (size_t)2 * GB_MAX_WGS * GB_PART_FLOATS * sizeof(float);
+}
+
+extern "C" int proteus_geo_attn_fwd_ws_check(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,
+                                             const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                             const float* O, const float* L, const void* workspace, size_t workspace_bytes,
+                                             int Z, int H, int N, int d_head, int tuning)
+{
+    const int rc = proteus_geo_attn_fwd_check(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    if (workspace_bytes != 0 && !workspace) return PROTEUS_ERR_NULL_POINTER;
+    if ((uintptr_t)workspace & 255) return PROTEUS_ERR_BAD_ALIGNMENT;
+    if (strides) {
+        GaStrides gs;
+        return strides_from(strides, Z, H, N, d_head, gs);
+    }
+    return PROTEUS_OK;
+}
+
+extern "C" int proteus_geo_attn_fwd_ws(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,
+                                       const float* coords, const float* sigma, const uint8_t* key_pad_mask,
+                                       float* O, float* L, void* workspace, size_t workspace_bytes,
+                                       int Z, int H, int N, int d_head, int tuning, void* stream)
+{
+    int rc = proteus_geo_attn_fwd_ws_check(Q, K, V, strides, coords, sigma, key_pad_mask, O, L, workspace, workspace_bytes,
+                                           Z, H, N, d_head, tuning);
+    if (rc != PROTEUS_OK) return rc;
+    GaStrides gs = contiguous_strides(H, N, d_head);
+    if (strides) {
+        rc = strides_from(strides, Z, H, N, d_head, gs);
+        if (rc != PROTEUS_OK) return rc;
+    }
+    return launch_attn(false, false, d_head, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning, nullptr, 0.f, 1.f, gs,
+                       reinterpret_cast<hipStream_t>(stream), workspace, workspace_bytes);
 }
 
 namespace {

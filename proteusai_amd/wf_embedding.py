@@ -116,13 +116,15 @@ class _wf_embedding(torch.autograd.Function):
     the reference."""
 
     @staticmethod
-    def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask):
+    def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask, recording=True):
         if magnitude_type not in (0, 1, 2, 3):
             raise AssertionError("magnitude_type must be one of 0, 1, 2, 3")
         if dropout_p != 0.0:
             raise NotImplementedError("dropout_p != 0 is not implemented; the module always passes 0.0")
         # the sums are what the backward for the wavenumbers consumes: without that gradient they are not computed
-        need = bool(ctx.needs_input_grad[1])
+        # (`recording`: was autograd recording when the operator was called?  Inside forward() it never is, and
+        # needs_input_grad repeats requires_grad whatever the mode: under no_grad / inference_mode no backward follows)
+        need = bool(recording and ctx.needs_input_grad[1])
         out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type, need_sums=need)
         if need:
             ctx.save_for_backward(cos_sums, sin_sums)
@@ -134,15 +136,15 @@ class _wf_embedding(torch.autograd.Function):
     def backward(ctx, dO):
         # (autograd also comes here when only another input, e.g. the coordinates, asks for a gradient: there is none to give)
         if not ctx.need:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         cos_sums, sin_sums = ctx.saved_tensors
         dk = we_backward(dO, cos_sums, sin_sums)
-        return None, dk.to(ctx.wn_dtype), None, None, None
+        return None, dk.to(ctx.wn_dtype), None, None, None, None
 
 
 def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None):
     """Same call as the reference's wf_embedding (isotropic/cuda/wf_embedding.py:18)."""
-    return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask)
+    return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask, torch.is_grad_enabled())
 
 
 def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tuning: int = 0, partials: bool = True):
@@ -200,10 +202,11 @@ class _wf_embedding_learnCB(torch.autograd.Function):
     coordinates, as in the reference."""
 
     @staticmethod
-    def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask):
+    def forward(ctx, coordsA, coordsB, cb_magnitudes, wavenumbers, mask, recording=True):
         # the per-token partial derivatives are computed only if autograd will ask for the gradient of one of the two
-        # scales (under no_grad / inference_mode it never does, whatever requires_grad says)
-        ctx.need = bool(ctx.needs_input_grad[2] or ctx.needs_input_grad[3])
+        # scales: `recording` says whether autograd was recording at the call (inside forward() it never is, and
+        # needs_input_grad repeats requires_grad whatever the mode: under no_grad / inference_mode no backward follows)
+        ctx.need = bool(recording and (ctx.needs_input_grad[2] or ctx.needs_input_grad[3]))
         out, d_cb, d_k = we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask, partials=ctx.need)
         if ctx.need:
             ctx.save_for_backward(d_cb, d_k)
@@ -213,18 +216,18 @@ class _wf_embedding_learnCB(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dO):
         if not ctx.need:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         d_cb, d_k = ctx.saved_tensors
         g_cb, g_k = we_aniso_backward(dO, d_cb if ctx.needs_input_grad[2] else None,
                                       d_k if ctx.needs_input_grad[3] else None)
         return (None, None, None if g_cb is None else g_cb.to(ctx.dtypes[0]),
-                None if g_k is None else g_k.to(ctx.dtypes[1]), None)
+                None if g_k is None else g_k.to(ctx.dtypes[1]), None, None)
 
 
 def wf_embedding_learnCB(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None):
     """Same call as the reference's anisotropic wf_embedding
     (anisotropic/cb_scaling/learnable_wavenumbers/cuda/wf_embedding.py:16)."""
-    return _wf_embedding_learnCB.apply(coordsA, coordsB, cb_magnitudes, wavenumbers, mask)
+    return _wf_embedding_learnCB.apply(coordsA, coordsB, cb_magnitudes, wavenumbers, mask, torch.is_grad_enabled())
 
 
 class WaveFunctionEmbedding(nn.Module):

@@ -180,8 +180,10 @@ def test_cfg4_shape_logits_match_the_cpu_statement_of_the_whole_stack(gpu, dtype
     (torch_oracle.encoder_forward_torch: dense torch attention and embedding oracles, pinned in
     tests/test_oracle_encoder.py), on every valid token.
 
-    Bars.  fp32 weights: the only low-precision steps are the attention's bf16 operands and probabilities (four
-    layers): rel-L2 over all valid logits <= 5e-3, max-abs <= 1 % of the logits' range.  bf16 weights (the
+    Bars (about twice what is measured: fp32 weights rel-L2 3.9e-3, worst token 2.5e-2, max-abs 0.85 % of the range;
+    bf16 weights 9.2e-3, 4.6e-2, 1.1 %).  fp32 weights: the only low-precision steps are the attention's bf16 operands
+    and probabilities (four layers): rel-L2 over all valid logits <= 8e-3, per token <= 5e-2, max-abs <= 2 % of the
+    logits' range.  bf16 weights (the
     configuration BASELINE names): every activation between two layers is rounded to bf16 (2^-9 relative, some 30
     roundings from the embedding to the head, which LayerNorm renormalises rather than damps): rel-L2 <= 2e-2, per
     token rel-L2 <= 8e-2 on every token, max-abs <= 4 % of the logits' range, and the arg-max amino acid agrees where
@@ -204,7 +206,7 @@ def test_cfg4_shape_logits_match_the_cpu_statement_of_the_whole_stack(gpu, dtype
     max_abs = float((got - want).abs().max())
     print(f"encoder at configs[3], {dtype}: rel-L2 {rel:.3e}, worst token {float(per_token.max()):.3e}, "
           f"max abs {max_abs:.3e} of a logit range of {span:.2f}", flush=True)
-    bars = {torch.float32: (5e-3, 3e-2, 0.01), torch.bfloat16: (2e-2, 8e-2, 0.04)}[dtype]
+    bars = {torch.float32: (8e-3, 5e-2, 0.02), torch.bfloat16: (2e-2, 8e-2, 0.04)}[dtype]
     assert rel <= bars[0], f"rel-L2 {rel:.3e}"
     assert float(per_token.max()) <= bars[1], f"worst token rel-L2 {float(per_token.max()):.3e}"
     assert max_abs <= bars[2] * span, f"max abs {max_abs:.3e}, range {span:.2f}"

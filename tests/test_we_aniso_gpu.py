@@ -181,7 +181,8 @@ def test_embedding_alone_equals_the_embedding_with_partials(gpu, tuning):
     assert rel_l2(y, full) <= 1e-6
     # learnable scales under no_grad / inference_mode: no gradient will be asked for, so the partial derivatives are not
     # produced either (the forward is called with partials=False)
-    import proteusai_amd.wf_embedding as wfe
+    import importlib
+    wfe = importlib.import_module("proteusai_amd.wf_embedding")     # (the package attribute of that name is the operator)
     seen = []
     real = wfe.we_aniso_forward
 

@@ -121,6 +121,34 @@ def test_without_sums_the_embedding_is_unchanged(gpu):
             assert torch.equal(full, lean), f"variant {name}, N={N}"
 
 
+def test_operator_computes_the_sums_only_when_a_backward_can_follow(gpu):
+    # the autograd operator asks for the sums (what its backward consumes) only when autograd is recording and the
+    # wavenumbers want a gradient: not under no_grad / inference_mode, whatever requires_grad says
+    import importlib
+    wfe = importlib.import_module("proteusai_amd.wf_embedding")       # (the package attribute of that name is the operator)
+    coords, wn = synth.we_inputs(200, seed=3, batch=2, d_model=32)
+    c, w = coords.to(gpu), wn.to(gpu).requires_grad_(True)
+    seen, real = [], wfe.we_forward
+
+    def spy(*args, **kwargs):
+        seen.append(kwargs.get("need_sums"))
+        return real(*args, **kwargs)
+    wfe.we_forward = spy
+    try:
+        with torch.no_grad():
+            y0 = pa.wf_embedding(c, w)
+        with torch.inference_mode():
+            pa.wf_embedding(c, w)
+        y1 = pa.wf_embedding(c, w)
+        y2 = pa.wf_embedding(c, w.detach())
+    finally:
+        wfe.we_forward = real
+    assert seen == [False, False, True, False]
+    assert y1.requires_grad and not y0.requires_grad and not y2.requires_grad and torch.equal(y0, y1.detach())
+    y1.sum().backward()
+    assert w.grad is not None and torch.isfinite(w.grad).all()
+
+
 def test_masks(gpu):
     N = 333
     coords, wn = synth.we_inputs(N, seed=5, batch=4, d_model=64)
