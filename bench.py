@@ -470,9 +470,9 @@ def main():
                            "valid lengths uniform in [2048, 4096], the rest padded (BASELINE.json configs[2])",
                "ms": ms3, "lengths": [int(x) for x in lens], "dtype": "bf16",
                "tflops_useful": useful / (ms3 * 1e-3) / 1e12, "tflops_dense_equivalent": dense / (ms3 * 1e-3) / 1e12,
-               "entry_point": "proteus_geo_attn_fwd_ws (plan + balanced persistent grid + gated plain grid: three launches)",
+               "entry_point": "proteus_geo_attn_fwd_ws (plan kernel + balanced persistent grid: two launches)",
                "ms_plain_grid": ms3_plain,
-               "roofline": {"kernel": "geo_attn_plan_kernel + geo_attn_fwd_balanced_kernel + geo_attn_fwd_pipe_kernel (gated)",
+               "roofline": {"kernel": "geo_attn_plan_kernel + geo_attn_fwd_balanced_kernel",
                             "bound": "mfma", "achieved": useful / (ms3 * 1e-3) / 1e12,
                             "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
                             "frac": useful / (ms3 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,

@@ -275,8 +275,8 @@ int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint1
  *   tuning       0 = automatic: the balanced schedule for N > 1024 and at least 24576 (item, key tile) steps of the full batch;
  *                8 = the balanced schedule wherever it is possible (d_head = 64, Z <= 256, fewer than 2^30 steps);
  *                proteus_geo_attn_fwd_workspace_bytes returns 0 where the given tuning does not take it
- * Launches (balanced path): a plan kernel, the persistent grid, and the plain grid, which returns at once unless a
- * query tile's tokens lie too far apart for the matrix-core distances (then it does the whole batch instead).
+ * Launches (balanced path): a plan kernel and the persistent grid (which falls back to direct vector-ALU distances,
+ * whole items in turn, if a query tile's tokens lie too far apart for the matrix-core distances).
  */
 size_t proteus_geo_attn_fwd_workspace_bytes(int Z, int H, int N, int d_head, int tuning);
 int proteus_geo_attn_fwd_ws(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,

@@ -56,7 +56,7 @@ namespace {
 #include "geo_attn_fwd_pipe.inc"
 
 // True if the plan of a padded batch (see geo_attn_plan_kernel) marks a query tile whose tokens spread too far for
-// the matrix-core distances: then the balanced kernel leaves the launch to the plain grid.
+// the matrix-core distances: then the balanced kernel runs the direct-distance body instead.
 // (`any_wide`: an int of the workgroup's LDS, free at that point)
 __device__ __forceinline__ bool ga_plan_has_wide_tile(const int* __restrict__ wide, const int n, int& any_wide) {
     if (threadIdx.x == 0) any_wide = 0;
@@ -72,19 +72,16 @@ __device__ __forceinline__ bool ga_plan_has_wide_tile(const int* __restrict__ wi
 
 // The pipelined body over the first half of a doubled grid, the direct-distance body (for workgroups whose
 // queries are spread too widely for the matrix-core distances) over the second; take_all: the pipelined body alone.
-// gate != NULL: the launch follows a balanced one over the same batch and does the work only if that one declined
-// (a query tile too wide for the matrix-core distances: gate[0 .. gate_n) holds a non-zero flag).
 __global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                               const uint16_t* __restrict__ V, const float* __restrict__ coords,
                               const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                               float* __restrict__ O, float* __restrict__ L,
                               const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs, const int take_all,
-                              const int* __restrict__ gate, const int gate_n, const int num_cus,
+                              const int num_cus,
                               const GaStrides st)
 {
     extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
-    if (gate && !ga_plan_has_wide_tile(gate, gate_n, reinterpret_cast<PipeSmem*>(ga_dyn_smem)->n_eff)) return;
     const int id = (int)blockIdx.x;
     if (id < n_wgs)
         // (workgroups are handed to the compute units in turn: num_cus apart they share one)
@@ -196,7 +193,17 @@ void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t
     int*       counters  = plan + (size_t)2 * Z * nqt;
 
     // ---- the plan every workgroup derives: lengths, steps before each batch item ----
-    if (ga_plan_has_wide_tile(wide, Z * nqt, bs.flag)) return; // the plain grid, launched next, does this batch
+    if (ga_plan_has_wide_tile(wide, Z * nqt, bs.flag)) {
+        // A query tile whose tokens lie too far apart for the matrix-core distances of the pipelined body (an extended
+        // chain): this batch is done with the direct-distance body instead, whole items in turn, no parts.
+        static_assert(sizeof(Smem) <= sizeof(BalSmem), "the direct-distance body's LDS fits");
+        for (int item = (int)blockIdx.x; item < Z * H * nqt; item += G) {
+            __syncthreads();
+            geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), item, Q, K, V, coords, sigma, key_pad, O, L,
+                                              H, N, Z * H, nqt, 1, nullptr, 0.f, 1.f, st);
+        }
+        return;
+    }
     for (int z = tid; z < Z; z += GA_THREADS) {
         int last = 0;
         for (int qt = 0; qt < nqt; ++qt) last = max(last, tile_last[(size_t)z * nqt + qt]);
@@ -385,7 +392,7 @@ int device_cus(int* cus_out) {
 
 int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                      const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, bool take_all,
-                     const int* gate, int gate_n, const GaStrides& gs, hipStream_t st)
+                     const GaStrides& gs, hipStream_t st)
 {
     static std::atomic<unsigned long long> allowed{0ull};
     const int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel), GA_PIPE_LDS, allowed);
@@ -398,7 +405,7 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
     const int rc2 = device_cus(&cus);
     if (rc2 != (int)hipSuccess) return rc2;
     hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
-                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gate, gate_n, cus, gs);
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, cus, gs);
     return (int)hipGetLastError();
 }
 
@@ -429,7 +436,7 @@ bool balanced_applies(const uint8_t* key_pad_mask, int Z, int H, int N, int d_he
     return forced || (N > 1024 && steps >= 48L * GB_MAX_WGS);
 }
 
-// Plan, balanced launch, and the plain grid gated on the plan (it runs only if the balanced launch declined).
+// The plan and the persistent grid.
 int launch_attn_balanced(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
                          const uint8_t* key_pad_mask, float* O, float* L, void* workspace, int Z, int H, int N,
                          const GaStrides& gs, hipStream_t st)
@@ -446,9 +453,7 @@ int launch_attn_balanced(const uint16_t* Q, const uint16_t* K, const uint16_t* V
     hipLaunchKernelGGL(geo_attn_plan_kernel, dim3(nqt, Z), dim3(GA_THREADS), 0, st, coords, sigma, key_pad_mask, plan, Z, H, N, nqt);
     hipLaunchKernelGGL(geo_attn_fwd_balanced_kernel, dim3(G), dim3(GA_THREADS), sizeof(BalSmem), st,
                        Q, K, V, coords, sigma, key_pad_mask, O, L, plan, parts, Z, H, N, nqt, gs);
-    rc = (int)hipGetLastError();
-    if (rc != (int)hipSuccess) return rc;
-    return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, false, plan + (size_t)Z * nqt, Z * nqt, gs, st);
+    return (int)hipGetLastError();
 }
 
 // d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
@@ -478,7 +483,7 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
     const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
     if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
-        return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, nullptr, 0, gs, st);
+        return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
     return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
 }

@@ -133,19 +133,32 @@ def test_cfg3_shape_takes_the_balanced_schedule_automatically(gpu):
     check_oracle(auto, Q, K, V, coords, sigma, mask, rows, "cfg3")
 
 
-def test_tokens_too_far_apart_for_the_matrix_core_distances_go_to_the_plain_grid(gpu):
+def test_tokens_too_far_apart_for_the_matrix_core_distances_take_direct_distances(gpu):
     # a straight chain: the 256 tokens of a query tile span 970 A, far beyond what the matrix-core distances of the
-    # pipelined body resolve at sigma = 3 A.  The plan marks the tiles, the balanced launch declines and the plain grid
-    # (with its direct-distance body) does the batch within the same call.
+    # pipelined body resolve at sigma = 3 A.  The plan marks the tiles and the persistent grid runs the direct-distance
+    # body over whole items instead.
     Z, H, N = 2, 2, 1300
     Q, K, V, _, sigma, g = make(11, Z, H, N)
     coords = torch.zeros(Z, N, 3)
     coords[:, :, 0] = 3.8 * torch.arange(N)
     mask, lens = tail_mask(Z, N, g, 700)
     bal = run(gpu, Q, K, V, coords, sigma, mask, BALANCED)
-    plain = run(gpu, Q, K, V, coords, sigma, mask, PLAIN)
-    assert np.array_equal(bal[0], plain[0]) and np.array_equal(bal[1], plain[1])      # the same kernel did both
+    check_against_plain(bal, run(gpu, Q, K, V, coords, sigma, mask, PLAIN), "straight chain")
+    direct = run(gpu, Q, K, V, coords, sigma, mask, 2)              # direct distances on the plain grid (the launcher's tile shape)
+    assert np.abs(bal[0] - direct[0]).max() <= 2e-3 and np.array_equal(np.isneginf(bal[1]), np.isneginf(direct[1]))
     check_oracle(bal, Q, K, V, coords, sigma, mask, None, "straight chain")
+    # more items than persistent workgroups: every workgroup takes several in turn
+    Z, H, N = 5, 16, 2100
+    Q = (torch.randn(Z, H, N, 64, generator=g)).bfloat16()
+    K = (torch.randn(Z, H, N, 64, generator=g)).bfloat16()
+    V = torch.randn(Z, H, N, 64, generator=g).bfloat16()
+    coords = torch.zeros(Z, N, 3)
+    coords[:, :, 1] = 3.8 * torch.arange(N)
+    sigma = synth.log_spaced_sigma(H)
+    mask, lens = tail_mask(Z, N, g, 900)
+    bal = run(gpu, Q, K, V, coords, sigma, mask, BALANCED)
+    rows = np.unique(np.concatenate([np.random.default_rng(5).choice(N, 40, replace=False), [0, 255, 256, N - 1]])).astype(np.int32)
+    check_oracle(bal, Q, K, V, coords, sigma, mask, rows, "straight chain, 720 items")
 
 
 def test_raw_c_abi_strided_operands_no_lse_workspace_canary_and_reuse(gpu):
