@@ -141,6 +141,27 @@ def test_ragged_batch_of_long_sequences(gpu):
     compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "ragged N=1024")
 
 
+def test_padded_batches_handed_out_longest_first(gpu):
+    # The workgroups of a padded batch take the own tiles of the longest sequence first (up to 64 batch items): every
+    # (item, head, own tile) must still be done exactly once.  Equal lengths, an empty item, lengths on and beside the
+    # borders of the 128-token own tiles, a head count that does not divide 8, rows that are not multiples of 16 bytes.
+    N = 400
+    Q, K, V, dO, coords, sigma, _ = make(11, 7, 3, N)
+    mask = torch.zeros(7, N, dtype=torch.bool)
+    for z, n in enumerate((400, 10, 400, 0, 129, 128, 257)):
+        mask[z, n:] = True
+    a = (Q, K, V, dO, coords, sigma, mask)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "longest first")
+    # more items than are ranked: the launch order is kept
+    N = 130
+    Q, K, V, dO, coords, sigma, _ = make(12, 66, 1, N)
+    mask = torch.zeros(66, N, dtype=torch.bool)
+    for z in range(66):
+        mask[z, (z * 37) % 131:] = True
+    a = (Q, K, V, dO, coords, sigma, mask)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "66 items")
+
+
 def test_padded_content_cannot_matter(gpu):
     Q, K, V, dO, coords, sigma, mask = make(2, 2, 4, 260, maskfrac=0.3)
     got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask)
