@@ -495,6 +495,7 @@ def main():
         _, bms3 = time_launches(torch, bwd3_step, 20)
         leg["backward_ms"] = bms3
         leg["backward_tflops_useful_5_products"] = 2.5 * useful / (bms3 * 1e-3) / 1e12
+        leg["backward_frac"] = 2.5 * useful / (bms3 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS
         del dO3, D3, dQ3, dK3, dV3
         if not args.no_cpu:
             dt, runs = cpu_timed(lambda: torch_oracle.geo_attn_torch(Q3, K3, V3, c3, sg3, m3), 20.0, 3)
