@@ -259,40 +259,50 @@ void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t
             if (tid == 0) bs.flag = (nparts == 1) ? 1 : (atomicAdd(&counters[((size_t)z * nqt + qt) * H + h], 1) == nparts - 1);
             __syncthreads();
             if (bs.flag) {
-                // the last part of the item to finish adds them up, in the registers' layout: with M the largest
-                // reference among the parts that saw a key, O = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p.
-                // (The loads of a part are issued together: one round trip to memory per part and pass.)
+                // the last part of the item to finish adds them up, in the registers' layout and in share order:
+                // O = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M the largest reference among the parts
+                // that saw a key, kept as a running maximum (what has been added is rescaled when it grows).  The
+                // parts are taken two at a time, all loads of a pair issued together: one round trip to memory
+                // per pair and query block.
                 const int wave = tid >> 6, lane = tid & 63, half = lane >> 5, col = lane & 31;
                 float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
                 const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
 #pragma unroll 1
                 for (int bq = 0; bq < 2; ++bq) {
                     const int mlo = gp_part_ml_offset(wave, bq, col);
-                    float M = -INFINITY;
-                    for (int j = first_g; j <= last_g; ++j) {
-                        const floatx2 ml = __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(gp_part_rsrc(slot_of(j)), mlo, 0, GP_SC1));
-                        if (ml[1] > 0.f) M = fmaxf(M, ml[0]);
-                    }
-                    float l = 0.f;
+                    float M = -INFINITY, l = 0.f;
                     float acc[32];
 #pragma unroll
                     for (int r = 0; r < 32; ++r) acc[r] = 0.f;
-                    for (int j = first_g; j <= last_g; ++j) {
-                        const __amdgpu_buffer_rsrc_t rp = gp_part_rsrc(slot_of(j));
-                        const gp_uint2v rml = __builtin_amdgcn_raw_buffer_load_b64(rp, mlo, 0, GP_SC1);
-                        uint4v raw[8];
-#pragma unroll
-                        for (int q4 = 0; q4 < 8; ++q4)
-                            raw[q4] = __builtin_amdgcn_raw_buffer_load_b128(rp, gp_part_o_offset(wave, bq, q4 >> 2, q4 & 3, lane), 0, GP_SC1);
-                        const floatx2 ml = __builtin_bit_cast(floatx2, rml);
-                        const float w = (ml[1] > 0.f) ? __builtin_amdgcn_exp2f(ml[0] - M) : 0.f;
-                        l = __builtin_fmaf(w, ml[1], l);
+#pragma unroll 1
+                    for (int j = first_g; j <= last_g; j += 2) {
+                        const bool two = j + 1 <= last_g;
+                        const __amdgpu_buffer_rsrc_t rpa = gp_part_rsrc(slot_of(j));
+                        const __amdgpu_buffer_rsrc_t rpb = gp_part_rsrc(slot_of(two ? j + 1 : j));
+                        const gp_uint2v rmla = __builtin_amdgcn_raw_buffer_load_b64(rpa, mlo, 0, GP_SC1);
+                        const gp_uint2v rmlb = __builtin_amdgcn_raw_buffer_load_b64(rpb, mlo, 0, GP_SC1);
+                        uint4v rawa[8], rawb[8];
 #pragma unroll
                         for (int q4 = 0; q4 < 8; ++q4) {
-                            const floatx4 v = __builtin_bit_cast(floatx4, raw[q4]);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[4 * q4 + e] = __builtin_fmaf(w, v[e], acc[4 * q4 + e]);
+                            const int off = gp_part_o_offset(wave, bq, q4 >> 2, q4 & 3, lane);
+                            rawa[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpa, off, 0, GP_SC1);
+                            rawb[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpb, off, 0, GP_SC1);
                         }
+                        const floatx2 mla = __builtin_bit_cast(floatx2, rmla), mlb = __builtin_bit_cast(floatx2, rmlb);
+                        const bool ua = mla[1] > 0.f, ub = two && mlb[1] > 0.f;          // the part saw a key of this query
+                        const float Mn = fmaxf(M, fmaxf(ua ? mla[0] : -INFINITY, ub ? mlb[0] : -INFINITY));
+                        const float sc = (M > -INFINITY) ? __builtin_amdgcn_exp2f(M - Mn) : 0.f;
+                        const float wa = ua ? __builtin_amdgcn_exp2f(mla[0] - Mn) : 0.f;
+                        const float wb = ub ? __builtin_amdgcn_exp2f(mlb[0] - Mn) : 0.f;
+                        l = __builtin_fmaf(wb, mlb[1], __builtin_fmaf(wa, mla[1], l * sc));
+#pragma unroll
+                        for (int q4 = 0; q4 < 8; ++q4) {
+                            const floatx4 va = __builtin_bit_cast(floatx4, rawa[q4]), vb = __builtin_bit_cast(floatx4, rawb[q4]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                acc[4 * q4 + e] = __builtin_fmaf(wb, vb[e], __builtin_fmaf(wa, va[e], acc[4 * q4 + e] * sc));
+                        }
+                        M = Mn;
                     }
                     const int qi = qt * (GA_WAVES * 64) + wave * 64 + 32 * bq + col;
                     if (qi < N) {
