@@ -463,6 +463,14 @@ def main():
                 _lib.check(rc, "proteus_geo_attn_fwd_ws")
         _, ms3 = time_launches(torch, attn3_step, 50)
         _, ms3_plain = time_launches(torch, lambda: attn_forward_into(q3, k3, v3, c3d, s3d, m3d, O3, L3), 50)
+
+        def attn3_balanced_step():          # the other schedule for padded batches (equal shares of steps, persistent grid)
+            rc = lib.proteus_geo_attn_fwd_ws(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), None, c3d.data_ptr(), s3d.data_ptr(),
+                                             m3u.data_ptr(), O3.data_ptr(), L3.data_ptr(), ws3.data_ptr(), ws3_bytes,
+                                             4, 8, 4096, 64, 8, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_geo_attn_fwd_ws")
+        _, ms3_balanced = time_launches(torch, attn3_balanced_step, 50)
         lens = (~m3).sum(dim=1).double()
         useful = 4.0 * 8 * 64 * float((lens * lens).sum())
         dense = 4.0 * 4 * 8 * 64 * 4096 * 4096
@@ -470,9 +478,9 @@ def main():
                            "valid lengths uniform in [2048, 4096], the rest padded (BASELINE.json configs[2])",
                "ms": ms3, "lengths": [int(x) for x in lens], "dtype": "bf16",
                "tflops_useful": useful / (ms3 * 1e-3) / 1e12, "tflops_dense_equivalent": dense / (ms3 * 1e-3) / 1e12,
-               "entry_point": "proteus_geo_attn_fwd_ws (plan kernel + balanced persistent grid: two launches)",
-               "ms_plain_grid": ms3_plain,
-               "roofline": {"kernel": "geo_attn_plan_kernel + geo_attn_fwd_balanced_kernel",
+               "entry_point": "proteus_geo_attn_fwd_ws (plan kernel + split-items grid: two launches)",
+               "ms_plain_grid": ms3_plain, "ms_balanced_schedule": ms3_balanced,
+               "roofline": {"kernel": "geo_attn_plan_kernel + geo_attn_fwd_split_kernel",
                             "bound": "mfma", "achieved": useful / (ms3 * 1e-3) / 1e12,
                             "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
                             "frac": useful / (ms3 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
@@ -504,6 +512,31 @@ def main():
                                    "sample": f"the full workload, median of {runs} run(s), dense CPU PyTorch fp32 on the bf16-rounded inputs, {dt:.1f} s"}
         result["cfg3_attn_b4_n4096_padded"] = leg
         del q3, k3, v3, O3, L3, ws3
+
+    # ---------------- one unpadded sequence that does not fill the chip: Z=1, H=8, N=8192 (not a BASELINE configuration) ----------------
+    if "attn" in legs:
+        Q1, K1, V1, c1, sg1, _ = synth.attn_inputs(1, 8, 8192, 64, seed=8)
+        q1, k1, v1, c1d, s1d = (t.to(dev) for t in (Q1, K1, V1, c1, sg1))
+        O1 = torch.empty(1, 8, 8192, 64, device=dev)
+        L1 = torch.empty(1, 8, 8192, device=dev)
+        ws1_bytes = lib.proteus_geo_attn_fwd_workspace_bytes(1, 8, 8192, 64, 0)
+        ws1 = torch.empty(max(ws1_bytes, 256), dtype=torch.uint8, device=dev)
+
+        def attn1_step():
+            rc = lib.proteus_geo_attn_fwd_ws(q1.data_ptr(), k1.data_ptr(), v1.data_ptr(), None, c1d.data_ptr(), s1d.data_ptr(),
+                                             None, O1.data_ptr(), L1.data_ptr(), ws1.data_ptr(), ws1_bytes, 1, 8, 8192, 64, 0, stream)
+            if rc != 0:
+                _lib.check(rc, "proteus_geo_attn_fwd_ws")
+        _, ms1 = time_launches(torch, attn1_step, 30)
+        _, ms1_plain = time_launches(torch, lambda: attn_forward_into(q1, k1, v1, c1d, s1d, None, O1, L1), 30)
+        flop1 = 4.0 * 8 * 64 * 8192.0 * 8192.0
+        result["geo_attn_single_sequence_n8192"] = {
+            "workload": "geometric attention forward Z=1 H=8 N=8192 d_head=64 bf16, no mask: 256 items for 512 workgroup slots "
+                        "(with a workspace every item is split into two parts)",
+            "ms": ms1, "ms_plain_grid": ms1_plain, "tflops": flop1 / (ms1 * 1e-3) / 1e12,
+            "frac": flop1 / (ms1 * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+            "frac_plain_grid": flop1 / (ms1_plain * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS}
+        del q1, k1, v1, O1, L1, ws1
 
     # ---------------- geometric attention forward, N=16384, H=8, d=64 (configs[4]) ----------------
     if "attn" in legs or "attn_bwd" in legs:

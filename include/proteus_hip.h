@@ -260,23 +260,32 @@ int proteus_geo_attn_fwd_check(const uint16_t* Q, const uint16_t* K, const uint1
                                int Z, int H, int N, int d_head, int tuning);
 
 /*
- * proteus_geo_attn_fwd with a caller-provided workspace, for batches that come with a padding mask (d_head = 64).
- * The reference's launch gives every (batch, head, query tile) one program whose key loop is as long as the sequence
- * (old/old_scripts/attn/geometric_attn.py:586-599), so a padded batch lasts as long as its longest sequence.  With a
- * workspace the work is cut into equal shares instead (key tiles of one item may go to several workgroups, whose
- * partial results meet in the workspace).  Same result as proteus_geo_attn_fwd to fp32 rounding of the final
- * normalisation (the partial sums of a query are added in a different order).
+ * proteus_geo_attn_fwd with a caller-provided workspace (d_head = 64).  The reference's launch gives every (batch,
+ * head, query tile) item one program whose key loop is as long as the sequence
+ * (old/old_scripts/attn/geometric_attn.py:586-599): a padded batch lasts as long as its longest sequence, and a batch
+ * with fewer items than the chip has workgroup slots leaves most of it idle.  With a workspace the key loop of an item
+ * may be cut into parts that go to several workgroups, whose partial results meet in the workspace (the last of an
+ * item's parts to finish adds them up, in a fixed order: the result does not depend on which one that is).  Same result
+ * as proteus_geo_attn_fwd up to the rounding of the probabilities (a part re-bases its softmax reference where the whole
+ * item would not).
  *   strides      as proteus_geo_attn_fwd_strided, or NULL for contiguous [Z,H,N,d_head] tensors
+ *   key_pad_mask may be NULL
  *   workspace    device memory, 256-byte aligned, workspace_bytes >= proteus_geo_attn_fwd_workspace_bytes(Z, H, N,
  *                d_head, tuning); not initialised by the caller, nothing kept in it between calls; calls that share
- *                one workspace must not overlap.  NULL / too small (or a shape for which
- *                proteus_geo_attn_fwd_workspace_bytes returns 0, or key_pad_mask == NULL): the call is
- *                proteus_geo_attn_fwd[_strided].
- *   tuning       0 = automatic: the balanced schedule for N > 1024 and at least 24576 (item, key tile) steps of the full batch;
- *                8 = the balanced schedule wherever it is possible (d_head = 64, Z <= 256, fewer than 2^30 steps);
- *                proteus_geo_attn_fwd_workspace_bytes returns 0 where the given tuning does not take it
- * Launches (balanced path): a plan kernel and the persistent grid (which falls back to direct vector-ALU distances,
- * whole items in turn, if a query tile's tokens lie too far apart for the matrix-core distances).
+ *                one workspace must not overlap.  NULL / too small, or a shape for which
+ *                proteus_geo_attn_fwd_workspace_bytes returns 0: the call is proteus_geo_attn_fwd[_strided].
+ *   tuning       0 = automatic: the split-items schedule (9) for a padded batch with N >= 1024 and at least 8192
+ *                    (item, key tile) steps in the full batch, and for an unpadded batch with N > 2048 and fewer than 512
+ *                    items (the size function answers for the shape alone, as if either could be the case);
+ *                9 = split items wherever possible (d_head = 64, Z <= 256, fewer than 2^30 steps): when the live items
+ *                    are fewer than the chip's workgroup slots, the longest are cut along the keys into equal parts
+ *                    until the parts fill the slots; parts are handed out longest first;
+ *                8 = the balanced schedule wherever possible (same limits): all (item, key tile) steps as one line, cut
+ *                    into equal shares for a persistent grid of two workgroups per compute unit;
+ *                proteus_geo_attn_fwd_workspace_bytes returns 0 where the given tuning takes neither
+ * Launches (both schedules): a plan kernel (last unpadded token of every query tile, arrival counters) and the grid,
+ * which falls back to direct vector-ALU distances, whole items in turn, if a query tile's tokens lie too far apart
+ * for the matrix-core distances.
  */
 size_t proteus_geo_attn_fwd_workspace_bytes(int Z, int H, int N, int d_head, int tuning);
 int proteus_geo_attn_fwd_ws(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const int64_t* strides,

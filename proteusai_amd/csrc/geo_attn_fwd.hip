@@ -176,6 +176,74 @@ void geo_attn_plan_kernel(const float* __restrict__ coords, const float* __restr
     for (int h = tid; h < H; h += GA_THREADS) counters[t * H + h] = 0;
 }
 
+
+// The last part of an item to finish adds the parts up, in the registers' layout and in part order:
+// O = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M the largest reference among the parts that saw a key, kept as a
+// running maximum (what has been added is rescaled when it grows).  The parts are taken two at a time, all loads of
+// a pair issued together: one round trip to memory per pair and query block.  slot_of(j): where part j lies.
+template <typename SlotOf>
+__device__ __forceinline__ void gb_merge_parts(const SlotOf& slot_of, const int first_g, const int last_g,
+                                   float* __restrict__ O, float* __restrict__ L, const uint8_t* __restrict__ key_pad,
+                                   const int z, const int h, const int zh, const int qt, const int N, const GaStrides& st)
+{
+    const int tid = (int)threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, half = lane >> 5, col = lane & 31;
+    float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
+    const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
+#pragma unroll 1
+    for (int bq = 0; bq < 2; ++bq) {
+        const int mlo = gp_part_ml_offset(wave, bq, col);
+        float M = -INFINITY, l = 0.f;
+        float acc[32];
+#pragma unroll
+        for (int r = 0; r < 32; ++r) acc[r] = 0.f;
+#pragma unroll 1
+        for (int j = first_g; j <= last_g; j += 2) {
+            const bool two = j + 1 <= last_g;
+            const __amdgpu_buffer_rsrc_t rpa = gp_part_rsrc(slot_of(j));
+            const __amdgpu_buffer_rsrc_t rpb = gp_part_rsrc(slot_of(two ? j + 1 : j));
+            const gp_uint2v rmla = __builtin_amdgcn_raw_buffer_load_b64(rpa, mlo, 0, GP_SC1);
+            const gp_uint2v rmlb = __builtin_amdgcn_raw_buffer_load_b64(rpb, mlo, 0, GP_SC1);
+            uint4v rawa[8], rawb[8];
+#pragma unroll
+            for (int q4 = 0; q4 < 8; ++q4) {
+                const int off = gp_part_o_offset(wave, bq, q4 >> 2, q4 & 3, lane);
+                rawa[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpa, off, 0, GP_SC1);
+                rawb[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpb, off, 0, GP_SC1);
+            }
+            const floatx2 mla = __builtin_bit_cast(floatx2, rmla), mlb = __builtin_bit_cast(floatx2, rmlb);
+            const bool ua = mla[1] > 0.f, ub = two && mlb[1] > 0.f;          // the part saw a key of this query
+            const float Mn = fmaxf(M, fmaxf(ua ? mla[0] : -INFINITY, ub ? mlb[0] : -INFINITY));
+            const float sc = (M > -INFINITY) ? __builtin_amdgcn_exp2f(M - Mn) : 0.f;
+            const float wa = ua ? __builtin_amdgcn_exp2f(mla[0] - Mn) : 0.f;
+            const float wb = ub ? __builtin_amdgcn_exp2f(mlb[0] - Mn) : 0.f;
+            l = __builtin_fmaf(wb, mlb[1], __builtin_fmaf(wa, mla[1], l * sc));
+#pragma unroll
+            for (int q4 = 0; q4 < 8; ++q4) {
+                const floatx4 va = __builtin_bit_cast(floatx4, rawa[q4]), vb = __builtin_bit_cast(floatx4, rawb[q4]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[4 * q4 + e] = __builtin_fmaf(wb, vb[e], __builtin_fmaf(wa, va[e], acc[4 * q4 + e] * sc));
+            }
+            M = Mn;
+        }
+        const int qi = qt * (GA_WAVES * 64) + wave * 64 + 32 * bq + col;
+        if (qi < N) {
+            const bool row_ok = l > 0.f && !(mz && mz[qi]);
+            const float inv_l = row_ok ? 1.0f / l : 0.f;
+            float* orow = Oh + (size_t)qi * (size_t)st.o[2];
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq)
+                    *reinterpret_cast<float4*>(orow + dt * 32 + 8 * gq + 4 * half) =
+                        make_float4(acc[dt * 16 + 4 * gq] * inv_l, acc[dt * 16 + 4 * gq + 1] * inv_l,
+                                    acc[dt * 16 + 4 * gq + 2] * inv_l, acc[dt * 16 + 4 * gq + 3] * inv_l);
+            if (L && half == 0) L[(size_t)zh * N + qi] = row_ok ? (M + __log2f(l)) * 0.69314718055994531f : -INFINITY;
+        }
+    }
+}
+
 __global__ __launch_bounds__(GA_THREADS, 2)
 void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                                   const uint16_t* __restrict__ V, const float* __restrict__ coords,
@@ -259,66 +327,7 @@ void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t
             if (tid == 0) bs.flag = (nparts == 1) ? 1 : (atomicAdd(&counters[((size_t)z * nqt + qt) * H + h], 1) == nparts - 1);
             __syncthreads();
             if (bs.flag) {
-                // the last part of the item to finish adds them up, in the registers' layout and in share order:
-                // O = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M the largest reference among the parts
-                // that saw a key, kept as a running maximum (what has been added is rescaled when it grows).  The
-                // parts are taken two at a time, all loads of a pair issued together: one round trip to memory
-                // per pair and query block.
-                const int wave = tid >> 6, lane = tid & 63, half = lane >> 5, col = lane & 31;
-                float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
-                const uint8_t* mz = key_pad ? key_pad + (size_t)z * N : nullptr;
-#pragma unroll 1
-                for (int bq = 0; bq < 2; ++bq) {
-                    const int mlo = gp_part_ml_offset(wave, bq, col);
-                    float M = -INFINITY, l = 0.f;
-                    float acc[32];
-#pragma unroll
-                    for (int r = 0; r < 32; ++r) acc[r] = 0.f;
-#pragma unroll 1
-                    for (int j = first_g; j <= last_g; j += 2) {
-                        const bool two = j + 1 <= last_g;
-                        const __amdgpu_buffer_rsrc_t rpa = gp_part_rsrc(slot_of(j));
-                        const __amdgpu_buffer_rsrc_t rpb = gp_part_rsrc(slot_of(two ? j + 1 : j));
-                        const gp_uint2v rmla = __builtin_amdgcn_raw_buffer_load_b64(rpa, mlo, 0, GP_SC1);
-                        const gp_uint2v rmlb = __builtin_amdgcn_raw_buffer_load_b64(rpb, mlo, 0, GP_SC1);
-                        uint4v rawa[8], rawb[8];
-#pragma unroll
-                        for (int q4 = 0; q4 < 8; ++q4) {
-                            const int off = gp_part_o_offset(wave, bq, q4 >> 2, q4 & 3, lane);
-                            rawa[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpa, off, 0, GP_SC1);
-                            rawb[q4] = __builtin_amdgcn_raw_buffer_load_b128(rpb, off, 0, GP_SC1);
-                        }
-                        const floatx2 mla = __builtin_bit_cast(floatx2, rmla), mlb = __builtin_bit_cast(floatx2, rmlb);
-                        const bool ua = mla[1] > 0.f, ub = two && mlb[1] > 0.f;          // the part saw a key of this query
-                        const float Mn = fmaxf(M, fmaxf(ua ? mla[0] : -INFINITY, ub ? mlb[0] : -INFINITY));
-                        const float sc = (M > -INFINITY) ? __builtin_amdgcn_exp2f(M - Mn) : 0.f;
-                        const float wa = ua ? __builtin_amdgcn_exp2f(mla[0] - Mn) : 0.f;
-                        const float wb = ub ? __builtin_amdgcn_exp2f(mlb[0] - Mn) : 0.f;
-                        l = __builtin_fmaf(wb, mlb[1], __builtin_fmaf(wa, mla[1], l * sc));
-#pragma unroll
-                        for (int q4 = 0; q4 < 8; ++q4) {
-                            const floatx4 va = __builtin_bit_cast(floatx4, rawa[q4]), vb = __builtin_bit_cast(floatx4, rawb[q4]);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                acc[4 * q4 + e] = __builtin_fmaf(wb, vb[e], __builtin_fmaf(wa, va[e], acc[4 * q4 + e] * sc));
-                        }
-                        M = Mn;
-                    }
-                    const int qi = qt * (GA_WAVES * 64) + wave * 64 + 32 * bq + col;
-                    if (qi < N) {
-                        const bool row_ok = l > 0.f && !(mz && mz[qi]);
-                        const float inv_l = row_ok ? 1.0f / l : 0.f;
-                        float* orow = Oh + (size_t)qi * (size_t)st.o[2];
-#pragma unroll
-                        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                            for (int gq = 0; gq < 4; ++gq)
-                                *reinterpret_cast<float4*>(orow + dt * 32 + 8 * gq + 4 * half) =
-                                    make_float4(acc[dt * 16 + 4 * gq] * inv_l, acc[dt * 16 + 4 * gq + 1] * inv_l,
-                                                acc[dt * 16 + 4 * gq + 2] * inv_l, acc[dt * 16 + 4 * gq + 3] * inv_l);
-                        if (L && half == 0) L[(size_t)zh * N + qi] = row_ok ? (M + __log2f(l)) * 0.69314718055994531f : -INFINITY;
-                    }
-                }
+                gb_merge_parts(slot_of, first_g, last_g, O, L, key_pad, z, h, zh, qt, N, st);
             }
         }
         a += k1 - k0;
@@ -340,9 +349,156 @@ void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t
     }
 }
 
+// ---------------- padded batches, second schedule: long items split, longest parts first ----------------
+//
+// The items (batch, head, query tile) of a padded batch differ in the length of their key loops.  When there are fewer
+// live items than the chip has workgroup slots (`cap`), the longest are split along the keys into equal parts until
+// the parts fill the slots: the smallest part length T for which sum_items ceil(c_item / T) <= cap.  Parts are numbered
+// longest first (sequences ranked by the length of their parts; within a sequence tile-major, the heads of a tile side
+// by side, so that with 8 heads each XCD keeps to one head) and workgroup p takes part p: the hardware hands the
+// workgroups out in this order.  An item that is not split is written directly; the parts of a split item meet as in
+// the balanced schedule (state in the workspace, a ticket per part, the last arriver adds them up in part order).
+// With at least `cap` live items nothing is split and the launch is the plain grid in longest-first order.
+__global__ __launch_bounds__(GA_THREADS, 2)
+void geo_attn_fwd_split_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                               const uint16_t* __restrict__ V, const float* __restrict__ coords,
+                               const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
+                               float* __restrict__ O, float* __restrict__ L,
+                               int* __restrict__ plan, float* __restrict__ parts,
+                               const int Z, const int H, const int N, const int nqt, const int cap, const int num_cus,
+                               const GaStrides st)
+{
+    extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
+    BalSmem& bs = *reinterpret_cast<BalSmem*>(ga_dyn_smem);
+    const int tid = (int)threadIdx.x;
+    const int G = (int)gridDim.x;
+    const int* tile_last = plan;
+    const int* wide      = plan + (size_t)Z * nqt;
+    int*       counters  = plan + (size_t)2 * Z * nqt;
+
+    if (ga_plan_has_wide_tile(wide, Z * nqt, bs.flag)) {
+        for (int item = (int)blockIdx.x; item < Z * H * nqt; item += G) {
+            __syncthreads();
+            geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), item, Q, K, V, coords, sigma, key_pad, O, L,
+                                              H, N, Z * H, nqt, 1, nullptr, 0.f, 1.f, st);
+        }
+        return;
+    }
+    // (the tables below live in the K ring until the part begins: order[r], count prefix[r], splits[r] per rank)
+    int* order  = reinterpret_cast<int*>(&bs.pipe.kring[0][0]);
+    int* splits = order + GB_MAX_Z;
+    for (int z = tid; z < Z; z += GA_THREADS) {
+        int last = 0;
+        for (int qt = 0; qt < nqt; ++qt) last = max(last, tile_last[(size_t)z * nqt + qt]);
+        bs.n_eff[z] = last;
+    }
+    if (tid == 0) bs.flag = 0x7fffffff;
+    __syncthreads();
+    // live items, steps, longest key loop
+    int items = 0, c_max = 0;
+    long steps = 0;
+    for (int z = 0; z < Z; ++z) {
+        const int ne = bs.n_eff[z];
+        const int nq = (ne + GA_THREADS - 1) / GA_THREADS, c = (ne + GA_BN - 1) / GA_BN;
+        items += H * nq; steps += (long)H * nq * c; c_max = max(c_max, c);
+    }
+    int T = max(c_max, 1);
+    if (items < cap && items > 0) {
+        // the smallest part length whose parts fit the slots; thread t tries T_min + t
+        const int T_min = max((int)((steps + cap - 1) / cap), 1);
+        const int Tt = T_min + tid;
+        if (Tt <= c_max) {
+            int n = 0;
+            for (int z = 0; z < Z; ++z) {
+                const int ne = bs.n_eff[z];
+                const int nq = (ne + GA_THREADS - 1) / GA_THREADS, c = (ne + GA_BN - 1) / GA_BN;
+                n += H * nq * ((c + Tt - 1) / Tt);
+            }
+            if (n <= cap) atomicMin(&bs.flag, Tt);
+        }
+        __syncthreads();
+        T = min(bs.flag, c_max);
+    }
+    // rank the sequences by the length of their parts (longest first), count their parts
+    for (int z = tid; z < Z; z += GA_THREADS) {
+        const int ne = bs.n_eff[z];
+        const int c = (ne + GA_BN - 1) / GA_BN;
+        const int s = max((c + T - 1) / T, 1), plen = (c + s - 1) / s;
+        int r = 0;
+        for (int u = 0; u < Z; ++u) {
+            const int cu = (bs.n_eff[u] + GA_BN - 1) / GA_BN;
+            const int su = max((cu + T - 1) / T, 1), pu = (cu + su - 1) / su;
+            r += (pu > plen || (pu == plen && u < z)) ? 1 : 0;
+        }
+        order[r] = z;
+        splits[r] = s;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int r = 0; r < Z; ++r) {
+            bs.prefix[r] = run;
+            const int ne = bs.n_eff[order[r]];
+            run += H * ((ne + GA_THREADS - 1) / GA_THREADS) * splits[r];
+        }
+        bs.prefix[Z] = run;
+    }
+    __syncthreads();
+    const int n_parts = bs.prefix[Z];
+    const int p = (int)blockIdx.x;
+    if (p < n_parts) {
+        int r = 0;
+        while (bs.prefix[r + 1] <= p) ++r;
+        r = __builtin_amdgcn_readfirstlane(r);
+        const int z = order[r], s = splits[r];
+        const int ne = bs.n_eff[z];
+        const int c = (ne + GA_BN - 1) / GA_BN, plen = (c + s - 1) / s;
+        const int base = bs.prefix[r];
+        const int idx = p - base;
+        // (the second half of a sequence's parts takes the heads in mirrored order: an XCD, which sees the workgroups
+        // whose number is its own modulo 8, then works on a head of small sigma and one of large sigma, few near tiles and many)
+        const int rest = idx / H, nq = (ne + GA_THREADS - 1) / GA_THREADS;
+        const int h = (2 * rest >= nq * s) ? H - 1 - idx % H : idx % H;
+        const int part = rest % s, qt = rest / s;
+        const int zh = z * H + h;
+        const int role = (p / num_cus) & 1;
+        __syncthreads();                                      // (the tables in the K ring have been read)
+        if (s == 1) {
+            geo_attn_fwd_pipe_part<false>(bs.pipe, zh, qt, 0, c, ne, nullptr, role, Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
+        } else {
+            auto slot_of = [&](const int j) -> float* { return parts + (size_t)(base + (qt * s + j) * H + h) * GB_PART_FLOATS; };
+            const int k0 = part * plen, k1 = min(c, k0 + plen);
+            const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, slot_of(part), role,
+                                                        Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
+            if (rc == 0) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (tid == 0) bs.flag = (atomicAdd(&counters[((size_t)z * nqt + qt) * H + h], 1) == s - 1);
+                __syncthreads();
+                if (bs.flag) gb_merge_parts(slot_of, 0, s - 1, O, L, key_pad, z, h, zh, qt, N, st);
+            }
+        }
+    }
+
+    // ---- query tiles behind the last unpadded token of their sequence: zeros, L = -inf ----
+    for (int e = (int)blockIdx.x; e < Z * H * nqt; e += G) {
+        const int z = e / (H * nqt), rem = e - z * (H * nqt);
+        const int h = rem / nqt, qt = rem - h * nqt;
+        if (qt * GA_THREADS < bs.n_eff[z]) continue;
+        float* Oh = O + (size_t)z * st.o[0] + (size_t)h * st.o[1];
+        const int chunk = tid & 15;
+        for (int ql = tid >> 4; ql < GA_THREADS; ql += GA_THREADS / 16) {
+            const int qi = qt * GA_THREADS + ql;
+            if (qi >= N) break;
+            *reinterpret_cast<float4*>(Oh + (size_t)qi * (size_t)st.o[2] + 4 * chunk) = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (L && chunk == 0) L[((size_t)z * H + h) * N + qi] = -INFINITY;
+        }
+    }
+}
+
 struct GaVariant { const char* name; };
 const GaVariant kVariants[] = { {"auto"}, {"dist_mfma"}, {"dist_valu"}, {"one_block_per_wave"}, {"two_blocks_per_wave"},
-                                {"pipelined"}, {"pipelined_dist_mfma"}, {"split_keys"}, {"balanced"} };
+                                {"pipelined"}, {"pipelined_dist_mfma"}, {"split_keys"}, {"balanced"}, {"split_items"} };
 constexpr int kNumVariants = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
 
 }  // namespace
@@ -433,17 +589,33 @@ int balanced_grid(int* G) {
     return (int)hipSuccess;
 }
 
-// Is the balanced schedule possible for this shape (a padding mask, the pipelined body's head dimension, lengths and
-// prefix sums that fit the workgroup's LDS and 31-bit arithmetic) and, unless `forced`, worth taking: sequences long
-// enough that a workgroup's share holds a few parts at most and each part many key tiles.  From the shape alone.
-bool balanced_applies(const uint8_t* key_pad_mask, int Z, int H, int N, int d_head, bool forced) {
-    if (!key_pad_mask || d_head != GA_D || Z > GB_MAX_Z) return false;
+// Are the schedules that cut items into parts possible for this shape (the pipelined body's head dimension, lengths
+// and prefix sums that fit the workgroup's LDS and 31-bit arithmetic)?  From the shape alone.
+bool padded_schedules_possible(const uint8_t* key_pad_mask, int Z, int H, int N, int d_head) {
+    (void)key_pad_mask;
+    if (d_head != GA_D || Z > GB_MAX_Z) return false;
     const long nqt = (N + GA_THREADS - 1) / GA_THREADS, c = (N + GA_BN - 1) / GA_BN;
-    const long steps = (long)Z * H * nqt * c;
-    if (steps >= (1L << 30)) return false;
-    // (measured: 4 x 8 x 4096 with lengths 2344-3702 168 -> 151 us, 2 x 8 x 8192 160 -> 136 us; 8 x 8 x 2048 with 32 steps per
-    // workgroup on a full batch 111 -> 128 us: every part of an item costs a prologue of about four key tiles' time)
-    return forced || (N > 1024 && steps >= 48L * GB_MAX_WGS);
+    return (long)Z * H * nqt * c < (1L << 30);
+}
+
+// The balanced schedule (equal shares of steps) runs only where the tuning asks for it.
+bool balanced_applies(const uint8_t* key_pad_mask, int Z, int H, int N, int d_head, bool forced) {
+    return forced && padded_schedules_possible(key_pad_mask, Z, H, N, d_head);
+}
+
+// The split-items schedule is what a padded batch gets by itself when a workspace comes with it and the pipelined
+// body is the right one: sequences of at least 1024 tokens and 8192 steps in the dense batch.  Measured against the plain
+// grid (which takes the templated body for masked batches up to N = 1024): 4 x 8 x 4096 with lengths 2344-3702
+// 164 -> 142 us, 2 x 8 x 8192 (3555, 4019) 165 -> 123 us, 16 x 8 x 1024 (159-1000) 72 -> 65 us, 8 x 8 x 2048 (1180-1985: nothing
+// to split) 107 -> 110 us; the encoder's 8 x 8 x 1024 (4096 steps) 34 -> 45 us, hence the threshold.
+bool split_applies(const uint8_t* key_pad_mask, int Z, int H, int N, int d_head, bool forced) {
+    if (!padded_schedules_possible(key_pad_mask, Z, H, N, d_head)) return false;
+    const long nqt = (N + GA_THREADS - 1) / GA_THREADS, c = (N + GA_BN - 1) / GA_BN;
+    if (forced) return true;
+    // without a mask every item is as long as the others: splitting pays where the items do not fill the chip's
+    // workgroup slots (Z = 1, H = 8: N = 4096 98 -> 80 us, N = 8192 256 -> 217 us; Z = 3, N = 3000 163 -> 147 us; N = 2048 48 -> 49 us)
+    if (!key_pad_mask) return N > 2048 && (long)Z * H * nqt < GB_MAX_WGS;
+    return N >= 1024 && (long)Z * H * nqt * c >= 8192;
 }
 
 // The plan and the persistent grid.
@@ -466,6 +638,30 @@ int launch_attn_balanced(const uint16_t* Q, const uint16_t* K, const uint16_t* V
     return (int)hipGetLastError();
 }
 
+// The plan and the grid of the split-items schedule: one workgroup per part, at least `cap` of them.
+int launch_attn_split(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords, const float* sigma,
+                      const uint8_t* key_pad_mask, float* O, float* L, void* workspace, int Z, int H, int N,
+                      const GaStrides& gs, hipStream_t st)
+{
+    static std::atomic<unsigned long long> allowed{0ull};
+    int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_split_kernel), sizeof(BalSmem), allowed);
+    if (rc != (int)hipSuccess) return rc;
+    int cap = 0, cus = 0;
+    rc = balanced_grid(&cap);
+    if (rc != (int)hipSuccess) return rc;
+    rc = device_cus(&cus);
+    if (rc != (int)hipSuccess) return rc;
+    const int nqt = (N + GA_THREADS - 1) / GA_THREADS;
+    const long items = (long)Z * H * nqt;
+    const unsigned grid = (unsigned)(items > cap ? items : cap);
+    int*   plan  = static_cast<int*>(workspace);
+    float* parts = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gb_parts_offset(Z, H, nqt));
+    hipLaunchKernelGGL(geo_attn_plan_kernel, dim3(nqt, Z), dim3(GA_THREADS), 0, st, coords, sigma, key_pad_mask, plan, Z, H, N, nqt);
+    hipLaunchKernelGGL(geo_attn_fwd_split_kernel, dim3(grid), dim3(GA_THREADS), sizeof(BalSmem), st,
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, plan, parts, Z, H, N, nqt, cap, cus, gs);
+    return (int)hipGetLastError();
+}
+
 // d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
 // the software-pipelined kernel runs (automatically for large grids of long sequences, or when the tuning asks).
 int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords,
@@ -473,18 +669,23 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st,
                 void* workspace = nullptr, size_t workspace_bytes = 0)
 {
-    const bool pipe_tuning = tuning == 5 || tuning == 6 || tuning == 8;
+    const bool pipe_tuning = tuning == 5 || tuning == 6 || tuning == 8 || tuning == 9;
     if (d_head == 32)
         return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,
                                               beta, min_rbf, max_rbf, gs, st);
     if (d_head == 128)
         return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,
                                                beta, min_rbf, max_rbf, gs, st);
-    // A padded batch of long sequences, with a workspace to exchange partial results in: the balanced schedule.
-    if (!legacy && (tuning == 0 || tuning == 8) && workspace && balanced_applies(key_pad_mask, Z, H, N, d_head, tuning == 8)
-        && workspace_bytes >= proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d_head, tuning))
-        return launch_attn_balanced(Q, K, V, coords, sigma, key_pad_mask, O, L, workspace, Z, H, N, gs, st);
-    if (tuning == 8) tuning = 0;
+    // A padded batch with a workspace to exchange partial results in: long items split and handed out longest first
+    // (by itself where it pays, see split_applies), or the balanced schedule where the tuning asks for it.
+    if (!legacy && workspace && workspace_bytes >= proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d_head, tuning) &&
+        proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d_head, tuning) > 0) {
+        if ((tuning == 0 || tuning == 9) && split_applies(key_pad_mask, Z, H, N, d_head, tuning == 9))
+            return launch_attn_split(Q, K, V, coords, sigma, key_pad_mask, O, L, workspace, Z, H, N, gs, st);
+        if (tuning == 8 && balanced_applies(key_pad_mask, Z, H, N, d_head, true))
+            return launch_attn_balanced(Q, K, V, coords, sigma, key_pad_mask, O, L, workspace, Z, H, N, gs, st);
+    }
+    if (tuning == 8 || tuning == 9) tuning = 0;
     // The pipelined kernel pays a longer prologue back from about 16 key tiles per workgroup on, and only where its
     // 256-query workgroups fill the chip twice: measured against the templated body it wins from 512 workgroups and
     // N = 1024 on (3-11 %), loses below (7-9 % at 256 workgroups of N = 1024, 6-10 % at N = 256 and 512).  A batch that
@@ -566,9 +767,11 @@ extern "C" int proteus_geo_attn_fwd(const uint16_t* Q, const uint16_t* K, const 
 extern "C" size_t proteus_geo_attn_fwd_workspace_bytes(int Z, int H, int N, int d_head, int tuning)
 {
     if (Z <= 0 || H <= 0 || N <= 0 || N > PROTEUS_ATTN_MAX_N || (long)Z * H > 65535) return 0;
-    if (tuning != 0 && tuning != 8) return 0;
+    if (tuning != 0 && tuning != 8 && tuning != 9) return 0;
     // (whether a mask will be passed is not known here: sized as if)
-    if (!balanced_applies(reinterpret_cast<const uint8_t*>(1), Z, H, N, d_head, tuning == 8)) return 0;
+    const uint8_t* some_mask = reinterpret_cast<const uint8_t*>(1);
+    if (tuning == 8 ? !balanced_applies(some_mask, Z, H, N, d_head, true)
+                    : !(split_applies(some_mask, Z, H, N, d_head, tuning == 9) || split_applies(nullptr, Z, H, N, d_head, tuning == 9))) return 0;
     const int nqt = (N + GA_THREADS - 1) / GA_THREADS;
     return gb_parts_offset(Z, H, nqt) + (size_t)2 * GB_MAX_WGS * GB_PART_FLOATS * sizeof(float);
 }

@@ -103,14 +103,16 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         return (O, L) if return_lse else O
     with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        ws_bytes = lib.proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d, int(tuning)) if (m is not None and not legacy) else 0
+        ws_bytes = lib.proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d, int(tuning)) if not legacy else 0
         if ws_bytes:
-            # a padded batch of long sequences: with a workspace the library cuts the work into equal shares instead of
-            # one workgroup per (batch, head, query tile), whose key loop is as long as its sequence
+            # long sequences: with a workspace the library may cut the key loop of a (batch, head, query tile) item into
+            # parts -- the long items of a padded batch, or all items of a batch too small to fill the chip -- instead
+            # of one workgroup per item (the size is asked for the shape alone; without a use for it the call is the
+            # plain one)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             rc = lib.proteus_geo_attn_fwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                              None if _is_plain(q, k, v, O) else _lib.stride_array(q, k, v, O),
-                                             c.data_ptr(), s.data_ptr(), m.data_ptr(), O.data_ptr(), L.data_ptr(),
+                                             c.data_ptr(), s.data_ptr(), None if m is None else m.data_ptr(), O.data_ptr(), L.data_ptr(),
                                              ws.data_ptr(), ws_bytes, Z, H, N, d, int(tuning), stream)
         elif not legacy and _is_plain(q, k, v, O):
             rc = lib.proteus_geo_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
