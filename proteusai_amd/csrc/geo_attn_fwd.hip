@@ -420,18 +420,20 @@ void geo_attn_fwd_split_kernel(const uint16_t* __restrict__ Q, const uint16_t* _
         T = min(bs.flag, c_max);
     }
     // rank the sequences by the length of their parts (longest first), count their parts
+    int* plen_of = splits + GB_MAX_Z;                // (by batch item, until the ranks are known)
     for (int z = tid; z < Z; z += GA_THREADS) {
-        const int ne = bs.n_eff[z];
-        const int c = (ne + GA_BN - 1) / GA_BN;
-        const int s = max((c + T - 1) / T, 1), plen = (c + s - 1) / s;
+        const int c = (bs.n_eff[z] + GA_BN - 1) / GA_BN;
+        const int s = max((c + T - 1) / T, 1);
+        plen_of[z] = (c + s - 1) / s;
+    }
+    __syncthreads();
+    for (int z = tid; z < Z; z += GA_THREADS) {
+        const int plen = plen_of[z];
         int r = 0;
-        for (int u = 0; u < Z; ++u) {
-            const int cu = (bs.n_eff[u] + GA_BN - 1) / GA_BN;
-            const int su = max((cu + T - 1) / T, 1), pu = (cu + su - 1) / su;
-            r += (pu > plen || (pu == plen && u < z)) ? 1 : 0;
-        }
+        for (int u = 0; u < Z; ++u) { const int pu = plen_of[u]; r += (pu > plen || (pu == plen && u < z)) ? 1 : 0; }
+        const int c = (bs.n_eff[z] + GA_BN - 1) / GA_BN;
         order[r] = z;
-        splits[r] = s;
+        splits[r] = max((c + T - 1) / T, 1);
     }
     __syncthreads();
     if (tid == 0) {

@@ -97,6 +97,7 @@ def test_library_takes_the_balanced_schedule_where_these_tests_expect_it():
     (5, 4, 2600, 300, 1.0),         # shares of a few tiles: parts of two or three items per workgroup
     (1, 4, 8192, 8192, 1.0),        # nothing padded: whole items, nothing to merge but a part per item
     (2, 2, 4100, 1, 4.0),           # lengths from 1 on, large logits (re-based references differ between parts)
+    (37, 1, 520, 1, 1.0),           # many short sequences of every length (equal ones too): their ranking, single heads
 ])
 def test_tail_padding_against_oracle_and_plain_grid(gpu, sched, Z, H, N, lo, qscale):
     Q, K, V, coords, sigma, g = make(Z * 1000 + N, Z, H, N, qscale)
