@@ -66,7 +66,7 @@ extern "C" {
  * backward entry point take `int operand_type` before `tuning` / `stream`; a caller built against an older header
  * would pass its tuning selector there).  The Python binding checks for an exact match when it loads the library.
  */
-#define PROTEUS_VERSION 300
+#define PROTEUS_VERSION 301
 int proteus_version(void);
 
 /* Human-readable text for a return code of any entry point. */
@@ -125,13 +125,36 @@ const char* proteus_we_variant_name(int tuning);
  *     out[z,i,2k], out[z,i,2k+1] = sum_j valid * m cos(k_k r), sum_j valid * m sin(k_k r)
  *     cos_sums, sin_sums         = sum_j valid * m r cos(k_k r), ... sin   (kernel.cu:237-238)
  * Any other magnitude_type returns PROTEUS_ERR_UNSUPPORTED.  The reference's
- * in-kernel dropout (dropout_p != 0, kernel.cu:227-232) draws a fresh seed per call
- * (isotropic/cuda/wf_embedding.py:48-49) and is not provided.
+ * in-kernel dropout is proteus_we_dropout_fwd.
  */
 int proteus_we_legacy_fwd(const float* coords, int coords_layout,
                           const float* wavenumbers, const uint8_t* mask,
                           float* out, float* cos_sums, float* sin_sums,
                           int Z, int N, int K, int magnitude_type, void* stream);
+
+/*
+ * The forward with the reference kernel's in-kernel dropout: the native entry's dropout_p and rng_seed
+ * (isotropic/cuda/wf_embedding_if.cpp:20-25; kernel.cu:27-46 the hash, :227-232 its use).  The term of
+ * (batch item z, observer i, source j, wavenumber k) is kept iff
+ *     float(hash5(z, i, j, k, rng_seed)) / float(UINT32_MAX) >= dropout_p
+ * and what is kept is divided by 1 - dropout_p; cos_sums / sin_sums carry the same mask and factor (they are what the
+ * backward for the wavenumbers contracts, so the gradient is that of the masked sum).  The hash is integer
+ * arithmetic: the mask is the reference's to the bit for the same seed (its wrapper draws a fresh seed per call,
+ * isotropic/cuda/wf_embedding.py:48-49; here the caller passes it).  i and j are token indices, k the index of
+ * the wavenumber.
+ *   magnitude_type 0 .. 3 as proteus_we_legacy_fwd; cos_sums and sin_sums are required
+ *   dropout_p      0 <= dropout_p < 1 (else PROTEUS_ERR_BAD_SHAPE); 0 keeps every term
+ * proteus_we_dropout_threshold: the smallest value of the hash that is kept for a given dropout_p (host only).
+ */
+int proteus_we_dropout_fwd(const float* coords, int coords_layout,
+                           const float* wavenumbers, const uint8_t* mask,
+                           float* out, float* cos_sums, float* sin_sums,
+                           int Z, int N, int K, int magnitude_type, float dropout_p, uint32_t rng_seed, void* stream);
+int proteus_we_dropout_fwd_check(const float* coords, int coords_layout,
+                                 const float* wavenumbers, const uint8_t* mask,
+                                 const float* out, const float* cos_sums, const float* sin_sums,
+                                 int Z, int N, int K, int magnitude_type, float dropout_p);
+uint32_t proteus_we_dropout_threshold(float dropout_p);
 
 /*
  * Anisotropic (C-beta scaled, learnable wavenumber) Wavefunction Embedding

@@ -74,6 +74,40 @@ def we(coords, wavenumbers, mask=None, rows=None, precision="f64", mag_type=1):
     return out, cs, ss
 
 
+def we_dropout(coords, wavenumbers, mask, dropout_p, seed, rows=None, mag_type=1):
+    """The embedding with the reference kernel's in-kernel dropout (isotropic/cuda/wf_embedding_kernel.cu:27-46,
+    :227-238) for an explicit 32-bit seed; float64 (out [Z,R,2K], cos_sums, sin_sums [Z,R,K])."""
+    c = np.ascontiguousarray(np.asarray(coords, dtype=np.float32))
+    w = np.ascontiguousarray(np.asarray(wavenumbers, dtype=np.float32))
+    Z, N, three = c.shape
+    assert three == 3 and mag_type in (0, 1, 2, 3)
+    K = int(w.shape[0])
+    m = None if mask is None else np.ascontiguousarray(np.asarray(mask).astype(np.uint8))
+    r, R = _rows(rows, N)
+    out = np.empty((Z, R, 2 * K), np.float64)
+    cs = np.empty((Z, R, K), np.float64)
+    ss = np.empty((Z, R, K), np.float64)
+    fn = lib().we_oracle_dropout_f64
+    fn.restype = None
+    fn(_p(c, ctypes.c_float), _p(w, ctypes.c_float), _p(m, ctypes.c_uint8), ctypes.c_int(Z), ctypes.c_int(N), ctypes.c_int(K),
+       ctypes.c_int(mag_type), ctypes.c_float(dropout_p), ctypes.c_uint32(int(seed) & 0xffffffff),
+       _p(r, ctypes.c_int), ctypes.c_int(R), _p(out, ctypes.c_double), _p(cs, ctypes.c_double), _p(ss, ctypes.c_double))
+    return out, cs, ss
+
+
+def we_hash5(a, b, c, d, seed):
+    fn = lib().we_oracle_hash5
+    fn.restype = ctypes.c_uint32
+    return int(fn(ctypes.c_int(a), ctypes.c_int(b), ctypes.c_int(c), ctypes.c_int(d), ctypes.c_uint32(int(seed) & 0xffffffff)))
+
+
+def we_dropout_keep(z, i, j, k, seed, dropout_p):
+    fn = lib().we_oracle_dropout_keep
+    fn.restype = ctypes.c_int
+    return bool(fn(ctypes.c_int(z), ctypes.c_int(i), ctypes.c_int(j), ctypes.c_int(k), ctypes.c_uint32(int(seed) & 0xffffffff),
+                   ctypes.c_float(dropout_p)))
+
+
 def we_aniso(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, rows=None):
     """coordsA, coordsB [Z,N,3], cb_magnitudes, wavenumbers [K], mask [Z,N] bool (True = padded).
 

@@ -1,6 +1,8 @@
 /*
  * TEST INFRASTRUCTURE -- CPU oracle of the isotropic Wavefunction Embedding.
  * Not part of the product; the product path never links or calls this file.
+ * PARITY UNPINNED: we_oracle_hash5 (the dropout hash at the end of this file; see its comment).  Everything else is
+ * pinned by tests/test_oracle_we.py and tests/test_oracle_we_dropout.py.
  *
  * Follows, line by line in meaning:
  *   tests/wf_embed/wf_embed.py:91-129                    (wf_embedding_torch, mag_type 1)
@@ -137,6 +139,79 @@ void we_oracle_mag_f64(const float* coords, const float* wn, const uint8_t* mask
             for (int k = 0; k < K; ++k) {
                 const double ph = d * (double)wn[k];
                 const double co = cos(ph), si = sin(ph);
+                o[2*k] += co * w; o[2*k+1] += si * w; pc[k] += co * w * d; ps[k] += si * w * d;
+            }
+        }
+    }
+}
+
+/*
+ * The reference kernel's in-kernel dropout (isotropic/cuda/wf_embedding_kernel.cu):
+ *   hash5(a, b, c, d, seed)                                              kernel.cu:27-41
+ *       h = seed
+ *       h ^= a * 0x85ebca6b + 0x9e3779b9;  h ^= b * 0xc2b2ae35 + 0x165667b1
+ *       h ^= c * 0x27d4eb2f + 0xd6e8feb8;  h ^= d * 0x85ebca6b + 0x1b873593      (32-bit unsigned arithmetic)
+ *       h = (h ^ (h >> 16)) * 0x85ebca6b;  h ^= h >> 13;  h = (h ^ (h >> 16)) * 0xc2b2ae35;  h ^= h >> 16
+ *     (the reference's own hash: its last line resembles MurmurHash3's 32-bit finalizer but has one more shift-xor
+ *      before the second multiply, so no published known answer applies.  Constants and order are restated from the
+ *      source; only the reference's CUDA kernel could tell a typing slip in them: PARITY UNPINNED for the hash.
+ *      The 32-bit arithmetic, the keep test and the sums are pinned in tests/test_oracle_we_dropout.py.)
+ *   keep(z, i, j, k) = float(hash5(z, i, j, k, seed)) / float(UINT32_MAX) >= dropout_p          kernel.cu:43-46
+ *   real = keep * real / (1 - dropout_p), imag likewise; the sums take real * dists, imag * dists   kernel.cu:227-238
+ * The sums over sources are taken in double; mask, zero-distance rule and weights as we_oracle_mag_f64.
+ */
+uint32_t we_oracle_hash5(int a, int b, int c, int d, uint32_t seed)
+{
+    uint32_t h = seed;
+    h ^= ((uint32_t)a * 0x85ebca6bu) + 0x9e3779b9u;
+    h ^= ((uint32_t)b * 0xc2b2ae35u) + 0x165667b1u;
+    h ^= ((uint32_t)c * 0x27d4eb2fu) + 0xd6e8feb8u;
+    h ^= ((uint32_t)d * 0x85ebca6bu) + 0x1b873593u;
+    h = (h ^ (h >> 16)) * 0x85ebca6bu;
+    h ^= (h >> 13);
+    h = (h ^ (h >> 16)) * 0xc2b2ae35u;
+    h ^= (h >> 16);
+    return h;
+}
+
+int we_oracle_dropout_keep(int z, int i, int j, int k, uint32_t seed, float dropout_p)
+{
+    const uint32_t h = we_oracle_hash5(z, i, j, k, seed);
+    const float normalized = (float)h / (float)UINT32_MAX;
+    return normalized >= dropout_p;
+}
+
+void we_oracle_dropout_f64(const float* coords, const float* wn, const uint8_t* mask, int Z, int N, int K,
+                           int mag_type, float dropout_p, uint32_t seed, const int* rows, int nrows,
+                           double* out, double* cs, double* ss)
+{
+    const double scale = 1.0 / (1.0 - (double)dropout_p);
+    #pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int z = 0; z < Z; ++z)
+    for (int rr = 0; rr < nrows; ++rr) {
+        const int i = rows ? rows[rr] : rr;
+        const float* c = coords + (size_t)z * N * 3;
+        const uint8_t* m = mask ? mask + (size_t)z * N : NULL;
+        double* o = out + ((size_t)z * nrows + rr) * 2 * K;
+        double* pc = cs + ((size_t)z * nrows + rr) * K;
+        double* ps = ss + ((size_t)z * nrows + rr) * K;
+        for (int k = 0; k < K; ++k) { o[2*k] = o[2*k+1] = pc[k] = ps[k] = 0.0; }
+        if (m && m[i]) continue;
+        const double xi = c[3*i], yi = c[3*i+1], zi = c[3*i+2];
+        for (int j = 0; j < N; ++j) {
+            if (m && m[j]) continue;
+            const double dx = xi - c[3*j], dy = yi - c[3*j+1], dz = zi - c[3*j+2];
+            const double d2 = dx*dx + dy*dy + dz*dz;
+            if (d2 == 0.0) continue;
+            const double d = sqrt(d2);
+            double w = 1.0;
+            if (mag_type == 1) w = 1.0 / d;
+            if (mag_type == 2) w = 1.0 / log2(d);
+            if (mag_type == 3) w = 1.0 / sqrt(d);
+            for (int k = 0; k < K; ++k) {
+                if (dropout_p != 0.0f && !we_oracle_dropout_keep(z, i, j, k, seed, dropout_p)) continue;
+                const double ph = d * (double)wn[k];
+                const double co = cos(ph) * scale, si = sin(ph) * scale;
                 o[2*k] += co * w; o[2*k+1] += si * w; pc[k] += co * w * d; ps[k] += si * w * d;
             }
         }

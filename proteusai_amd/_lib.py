@@ -11,14 +11,15 @@ LIB_PATH = os.path.join(HERE, "libproteus_hip.so")
 
 COORDS_SOA = 0
 COORDS_AOS = 1
-ABI_VERSION = 300                    # PROTEUS_VERSION of the include/proteus_hip.h these argument lists were written from
+ABI_VERSION = 301                    # PROTEUS_VERSION of the include/proteus_hip.h these argument lists were written from
 OPERAND_BF16, OPERAND_F16 = 0, 1     # PROTEUS_OPERAND_* of include/proteus_hip.h
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2   # PROTEUS_DTYPE_*
 
 # every symbol include/proteus_hip.h declares
 SYMBOLS = [
     "proteus_version", "proteus_strerror",
-    "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_num_variants", "proteus_we_variant_name",
+    "proteus_we_fwd", "proteus_we_fwd_check", "proteus_we_legacy_fwd", "proteus_we_dropout_fwd", "proteus_we_dropout_fwd_check",
+    "proteus_we_dropout_threshold", "proteus_we_num_variants", "proteus_we_variant_name",
     "proteus_we_aniso_fwd", "proteus_we_aniso_fwd_check", "proteus_we_aniso_num_variants", "proteus_we_aniso_variant_name",
     "proteus_we_bwd_workspace_bytes", "proteus_we_bwd", "proteus_we_bwd_check", "proteus_we_bwd_static", "proteus_we_aniso_bwd", "proteus_we_aniso_bwd_check",
     "proteus_geo_attn_fwd", "proteus_geo_attn_fwd_check", "proteus_geo_attn_legacy_fwd", "proteus_geo_attn_bwd",
@@ -58,6 +59,12 @@ def load():
     lib.proteus_we_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
     lib.proteus_we_legacy_fwd.restype = ci
     lib.proteus_we_legacy_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.proteus_we_dropout_fwd.restype = ci
+    lib.proteus_we_dropout_fwd.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ctypes.c_float, ctypes.c_uint32, vp]
+    lib.proteus_we_dropout_fwd_check.restype = ci
+    lib.proteus_we_dropout_fwd_check.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ctypes.c_float]
+    lib.proteus_we_dropout_threshold.restype = ctypes.c_uint32
+    lib.proteus_we_dropout_threshold.argtypes = [ctypes.c_float]
     lib.proteus_we_fwd_check.restype = ci
     lib.proteus_we_fwd_check.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci]
     lib.proteus_we_num_variants.restype = ci

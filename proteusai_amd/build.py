@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "libproteus_hip.so")
-SOURCES = ["abi.hip", "we_fwd.hip", "we_aniso_fwd.hip", "we_bwd.hip", "geo_attn_fwd.hip", "geo_attn_fwd_d32.hip", "geo_attn_fwd_d128.hip",
+SOURCES = ["abi.hip", "we_fwd.hip", "we_dropout_fwd.hip", "we_aniso_fwd.hip", "we_bwd.hip", "geo_attn_fwd.hip", "geo_attn_fwd_d32.hip", "geo_attn_fwd_d128.hip",
            "geo_attn_bwd.hip", "geo_attn_bwd_d32.hip", "geo_attn_bwd_d128.hip", "geo_attn_delta.hip", "add_layernorm.hip"]
 PROBE_LIB = os.path.join(HERE, "libproteus_probes.so")
 PROBE_SOURCES = ["probes.hip"]

@@ -14,10 +14,15 @@ from . import _lib
 from .cb_utils import get_coords
 
 
-def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: int = 1, need_sums: bool = True):
+def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: int = 1, need_sums: bool = True,
+               dropout_p: float = 0.0, rng_seed=None):
     """out, cos_sums, sin_sums = we_forward(coords [Z,N,3], wavenumbers [K], mask [Z,N] bool | None).
 
     need_sums=False (weight 1/r only) skips the sums, which only the backward uses: returns (out, None, None).
+    dropout_p != 0: the reference kernel's in-kernel dropout (isotropic/cuda/wf_embedding_kernel.cu:27-46, :227-232):
+    every (batch item, observer, source, wavenumber) term is kept or dropped by a hash of its four indices and
+    rng_seed (a 32-bit integer; None draws a fresh one per call, as isotropic/cuda/wf_embedding.py:48-49 does), what is
+    kept is divided by 1 - dropout_p, and the sums carry the same mask.
     magnitude_type: the weight of a source at distance r, 0: 1, 1: 1/r (default), 2: 1/log2(r),
     3: 1/sqrt(r) (isotropic/cuda/wf_embedding_kernel.cu:192-206); the sums carry the weight times r.
 
@@ -30,6 +35,9 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
         raise ValueError(f"coords must be of shape (batch, N, 3), not {tuple(coords.shape)}")
     if wavenumbers.dim() != 1:
         raise ValueError(f"wavenumbers must be of shape (K,), not {tuple(wavenumbers.shape)}")
+    dropout_p = float(dropout_p)
+    if not (0.0 <= dropout_p < 1.0):
+        raise ValueError(f"dropout_p must be in [0, 1), not {dropout_p}")
     if not coords.is_cuda:
         raise _lib.ProteusError("we_forward needs tensors on the GPU (there is no CPU path)")
     lib = _lib.load()
@@ -45,14 +53,21 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
             raise ValueError(f"mask must be of shape ({Z}, {N}), not {tuple(mask.shape)}")
         m = mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
     out = torch.empty(Z, N, 2 * K, dtype=torch.float32, device=dev)
-    need_sums = need_sums or magnitude_type != 1
+    need_sums = need_sums or magnitude_type != 1 or dropout_p != 0.0
     cos_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev) if need_sums else None
     sin_sums = torch.empty(Z, N, K, dtype=torch.float32, device=dev) if need_sums else None
     if Z == 0 or N == 0 or K == 0:
         return out, cos_sums, sin_sums
     with _lib.on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        if magnitude_type == 1:
+        if dropout_p != 0.0:
+            if rng_seed is None:
+                rng_seed = int(torch.randint(0, 2 ** 32, (1,), dtype=torch.int64).item())
+            rc = lib.proteus_we_dropout_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
+                                            None if m is None else m.data_ptr(),
+                                            out.data_ptr(), cos_sums.data_ptr(), sin_sums.data_ptr(),
+                                            Z, N, K, int(magnitude_type), dropout_p, int(rng_seed) & 0xffffffff, stream)
+        elif magnitude_type == 1:
             rc = lib.proteus_we_fwd(c.data_ptr(), _lib.COORDS_AOS, w.data_ptr(),
                                     None if m is None else m.data_ptr(),
                                     out.data_ptr(), cos_sums.data_ptr() if need_sums else None,
@@ -116,16 +131,15 @@ class _wf_embedding(torch.autograd.Function):
     the reference."""
 
     @staticmethod
-    def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask, recording=True):
+    def forward(ctx, coords, wavenumbers, magnitude_type, dropout_p, mask, recording=True, rng_seed=None):
         if magnitude_type not in (0, 1, 2, 3):
             raise AssertionError("magnitude_type must be one of 0, 1, 2, 3")
-        if dropout_p != 0.0:
-            raise NotImplementedError("dropout_p != 0 is not implemented; the module always passes 0.0")
         # the sums are what the backward for the wavenumbers consumes: without that gradient they are not computed
         # (`recording`: was autograd recording when the operator was called?  Inside forward() it never is, and
         # needs_input_grad repeats requires_grad whatever the mode: under no_grad / inference_mode no backward follows)
         need = bool(recording and ctx.needs_input_grad[1])
-        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type, need_sums=need)
+        out, cos_sums, sin_sums = we_forward(coords, wavenumbers, mask, magnitude_type=magnitude_type, need_sums=need,
+                                             dropout_p=dropout_p, rng_seed=rng_seed)
         if need:
             ctx.save_for_backward(cos_sums, sin_sums)
         ctx.need = need
@@ -136,15 +150,16 @@ class _wf_embedding(torch.autograd.Function):
     def backward(ctx, dO):
         # (autograd also comes here when only another input, e.g. the coordinates, asks for a gradient: there is none to give)
         if not ctx.need:
-            return None, None, None, None, None, None
+            return None, None, None, None, None, None, None
         cos_sums, sin_sums = ctx.saved_tensors
         dk = we_backward(dO, cos_sums, sin_sums)
-        return None, dk.to(ctx.wn_dtype), None, None, None, None
+        return None, dk.to(ctx.wn_dtype), None, None, None, None, None
 
 
-def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None):
-    """Same call as the reference's wf_embedding (isotropic/cuda/wf_embedding.py:18)."""
-    return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask, torch.is_grad_enabled())
+def wf_embedding(coords, wavenumbers, magnitude_type=1, dropout_p=0.0, mask=None, rng_seed=None):
+    """Same call as the reference's wf_embedding (isotropic/cuda/wf_embedding.py:18); rng_seed (not in the reference,
+    which draws one per call) fixes the dropout mask."""
+    return _wf_embedding.apply(coords, wavenumbers, magnitude_type, dropout_p, mask, torch.is_grad_enabled(), rng_seed)
 
 
 def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tuning: int = 0, partials: bool = True):

@@ -189,9 +189,16 @@ def test_operator_argument_errors_match_the_reference_surface():
         pa.wf_embedding(coords, torch.rand(4), magnitude_type=5)
     with pytest.raises(_lib.ProteusError):
         pa.wf_embedding(coords, torch.rand(4), magnitude_type=0)      # exists, but not on the CPU
-    with pytest.raises(NotImplementedError):
-        pa.wf_embedding(coords, torch.rand(4), dropout_p=0.1)
+    with pytest.raises(_lib.ProteusError):
+        pa.wf_embedding(coords, torch.rand(4), dropout_p=0.1)              # exists, but not on the CPU
+    with pytest.raises(ValueError):
+        pa.wf_embedding(coords, torch.rand(4), dropout_p=1.0)              # the reference would divide by zero
     lib = _lib.load()
+    # the dropout entry point validates before any HIP call
+    assert lib.proteus_we_dropout_fwd(0x1000, 0, 0x1000, None, 0x1000, 0x1000, 0x1000, 1, 8, 4, 1, 1.5, 7, None) == -2
+    assert lib.proteus_we_dropout_fwd(0x1000, 0, 0x1000, None, 0x1000, None, None, 1, 8, 4, 1, 0.5, 7, None) == -1
+    assert lib.proteus_we_dropout_fwd(0x1000, 0, 0x1000, None, 0x1000, 0x1000, 0x1000, 1, 8, 4, 9, 0.5, 7, None) == -7
+    assert lib.proteus_we_dropout_threshold(0.0) == 0 and lib.proteus_we_dropout_threshold(0.5) == 2 ** 31 - 64
     assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, 0x1000, 0x1000, 0x1000, 1, 8, 4, 4, None) == -7
     assert lib.proteus_we_legacy_fwd(0x1000, 0, 0x1000, None, None, 0x1000, 0x1000, 1, 8, 4, 2, None) == -1
     # the other source weights have no variant without the sums
