@@ -78,15 +78,13 @@ void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __
                               const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                               float* __restrict__ O, float* __restrict__ L,
                               const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs, const int take_all,
-                              const int num_cus,
                               const GaStrides st)
 {
     extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
     const int id = (int)blockIdx.x;
     if (id < n_wgs)
-        // (workgroups are handed to the compute units in turn: num_cus apart they share one)
         geo_attn_fwd_pipe_body(*reinterpret_cast<PipeSmem*>(ga_dyn_smem), id, Q, K, V, coords, sigma, key_pad, O, L,
-                               H, N, ZH, n_qtiles, take_all, (id / num_cus) & 1, st);
+                               H, N, ZH, n_qtiles, take_all, st);
     else
         geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), id - n_wgs, Q, K, V, coords, sigma, key_pad, O, L,
                                           H, N, ZH, n_qtiles, 0, nullptr, 0.f, 1.f, st);
@@ -317,7 +315,7 @@ void geo_attn_fwd_balanced_kernel(const uint16_t* __restrict__ Q, const uint16_t
             return parts + ((size_t)2 * j + second) * GB_PART_FLOATS;
         };
         float* mine = slot_of(g);
-        const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, mine, (2 * (int)blockIdx.x >= G) ? 1 : 0,
+        const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, mine,
                                                     Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
         if (rc == 0) {
             // The part was written with device-scope stores: once they have completed it is in memory for every
@@ -365,7 +363,7 @@ void geo_attn_fwd_split_kernel(const uint16_t* __restrict__ Q, const uint16_t* _
                                const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
                                float* __restrict__ O, float* __restrict__ L,
                                int* __restrict__ plan, float* __restrict__ parts,
-                               const int Z, const int H, const int N, const int nqt, const int cap, const int num_cus,
+                               const int Z, const int H, const int N, const int nqt, const int cap,
                                const GaStrides st)
 {
     extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
@@ -463,14 +461,13 @@ void geo_attn_fwd_split_kernel(const uint16_t* __restrict__ Q, const uint16_t* _
         const int h = (2 * rest >= nq * s) ? H - 1 - idx % H : idx % H;
         const int part = rest % s, qt = rest / s;
         const int zh = z * H + h;
-        const int role = (p / num_cus) & 1;
         __syncthreads();                                      // (the tables in the K ring have been read)
         if (s == 1) {
-            geo_attn_fwd_pipe_part<false>(bs.pipe, zh, qt, 0, c, ne, nullptr, role, Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
+            geo_attn_fwd_pipe_part<false>(bs.pipe, zh, qt, 0, c, ne, nullptr, Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
         } else {
             auto slot_of = [&](const int j) -> float* { return parts + (size_t)(base + (qt * s + j) * H + h) * GB_PART_FLOATS; };
             const int k0 = part * plen, k1 = min(c, k0 + plen);
-            const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, slot_of(part), role,
+            const int rc = geo_attn_fwd_pipe_part<true>(bs.pipe, zh, qt, k0, k1, ne, slot_of(part),
                                                         Q, K, V, coords, sigma, key_pad, O, L, H, N, 1, st);
             if (rc == 0) {
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -569,11 +566,8 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
     const int n_qtiles = (N + BM - 1) / BM;
     const int ZH = Z * H;
     const unsigned n_wgs = (unsigned)n_qtiles * (unsigned)ZH;
-    int cus = 0;
-    const int rc2 = device_cus(&cus);
-    if (rc2 != (int)hipSuccess) return rc2;
     hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
-                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, cus, gs);
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gs);
     return (int)hipGetLastError();
 }
 
@@ -648,10 +642,8 @@ int launch_attn_split(const uint16_t* Q, const uint16_t* K, const uint16_t* V, c
     static std::atomic<unsigned long long> allowed{0ull};
     int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_split_kernel), sizeof(BalSmem), allowed);
     if (rc != (int)hipSuccess) return rc;
-    int cap = 0, cus = 0;
+    int cap = 0;
     rc = balanced_grid(&cap);
-    if (rc != (int)hipSuccess) return rc;
-    rc = device_cus(&cus);
     if (rc != (int)hipSuccess) return rc;
     const int nqt = (N + GA_THREADS - 1) / GA_THREADS;
     const long items = (long)Z * H * nqt;
@@ -660,7 +652,7 @@ int launch_attn_split(const uint16_t* Q, const uint16_t* K, const uint16_t* V, c
     float* parts = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gb_parts_offset(Z, H, nqt));
     hipLaunchKernelGGL(geo_attn_plan_kernel, dim3(nqt, Z), dim3(GA_THREADS), 0, st, coords, sigma, key_pad_mask, plan, Z, H, N, nqt);
     hipLaunchKernelGGL(geo_attn_fwd_split_kernel, dim3(grid), dim3(GA_THREADS), sizeof(BalSmem), st,
-                       Q, K, V, coords, sigma, key_pad_mask, O, L, plan, parts, Z, H, N, nqt, cap, cus, gs);
+                       Q, K, V, coords, sigma, key_pad_mask, O, L, plan, parts, Z, H, N, nqt, cap, gs);
     return (int)hipGetLastError();
 }
 
