@@ -162,6 +162,23 @@ def test_padded_batches_handed_out_longest_first(gpu):
     compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "66 items")
 
 
+def test_backward_after_a_forward_that_cut_its_items_into_parts(gpu):
+    # N > 2048 and few items: the operator's forward splits every item along the keys (parts merged through a
+    # workspace) and hands the backward its O and logsumexp; masked as well (the long items of a padded batch)
+    from proteusai_amd import _lib
+    assert _lib.load().proteus_geo_attn_fwd_workspace_bytes(2, 2, 2304, 64, 0) > 0
+    a = make(31, 2, 2, 2304)
+    compare(gpu_grads(gpu, *a), reference_grads(*a), None, "unmasked, split forward")
+    Q, K, V, dO, coords, sigma, _ = make(32, 3, 2, 2304)
+    mask = torch.zeros(3, 2304, dtype=torch.bool)
+    mask[0, 2200:] = True
+    mask[1, 700:] = True
+    mask[2, 1500:] = True
+    a = (Q, K, V, dO, coords, sigma, mask)
+    assert _lib.load().proteus_geo_attn_fwd_workspace_bytes(3, 2, 2304, 64, 0) > 0
+    compare(gpu_grads(gpu, *a), reference_grads(*a), mask, "masked, split forward")
+
+
 def test_padded_content_cannot_matter(gpu):
     Q, K, V, dO, coords, sigma, mask = make(2, 2, 4, 260, maskfrac=0.3)
     got = gpu_grads(gpu, Q, K, V, dO, coords, sigma, mask)
