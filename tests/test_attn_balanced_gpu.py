@@ -274,3 +274,29 @@ def test_padded_schedules_replay_from_a_captured_graph(gpu, sched):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_random_long_batches_through_the_operator(gpu, case):
+    # what the operator does by itself (tuning 0: split items where the shape asks for it, the plain grid otherwise) and
+    # both schedules forced, on random shapes with tail padding, scattered padding or none, against the oracle on sampled rows
+    rng = np.random.default_rng(1000 + case)
+    Z, H = int(rng.integers(1, 6)), int(rng.choice([1, 2, 3, 4, 8]))
+    N = int(rng.integers(1024, 4200))
+    Q, K, V, coords, sigma, g = make(5000 + case, Z, H, N, qscale=float(rng.choice([0.5, 1.0, 2.0])))
+    sigma = torch.exp(torch.empty(H).uniform_(np.log(2.0), np.log(30.0), generator=g))
+    kind = case % 3
+    if kind == 0:
+        mask = None
+    elif kind == 1:
+        mask, _ = tail_mask(Z, N, g, 1)
+    else:
+        mask, _ = tail_mask(Z, N, g, N // 3)
+        mask |= torch.rand(Z, N, generator=g) < 0.1
+    rows = np.unique(np.concatenate([rng.choice(N, 48, replace=False), [0, 255, 256, N - 1]])).astype(np.int32)
+    what = f"case {case}: Z={Z} H={H} N={N} mask kind {kind}"
+    auto = run(gpu, Q, K, V, coords, sigma, mask, 0)
+    check_oracle(auto, Q, K, V, coords, sigma, mask, rows, what + " (automatic)")
+    for tuning in (BALANCED, SPLIT):
+        got = run(gpu, Q, K, V, coords, sigma, mask, tuning)
+        check_oracle(got, Q, K, V, coords, sigma, mask, rows, what + f" (tuning {tuning})")
