@@ -157,11 +157,14 @@ def check_backward(gpu, Q, K, V, dO, coords, sigma, mask, betas, lo, hi, dtype, 
         assert (err <= scalar_tol * mass + 1e-30).all(), f"{what} {name}: error / pair mass {(err / mass.clamp_min(1e-300)).max():.3e}"
 
 
+# (Z, H): a launch of few workgroups (at d <= 64 they own 64 tokens each, two waves per own block) and one of more than
+# 256 workgroups of 128 own tokens
+@pytest.mark.parametrize("ZH", [(2, 3), (5, 32)])
 @pytest.mark.parametrize("d", [32, 128])
 @pytest.mark.parametrize("N", [2, 65, 200, 333])
-def test_backward_readme_logits(gpu, d, N):
-    a = make(700 + N + d, 2, 3, N, d, torch.bfloat16, maskfrac=0.2 if N > 65 else 0.0)
-    check_backward(gpu, *a, None, 0.0, 1.0, torch.bfloat16, 2.0 ** -9, f"d={d} N={N}")
+def test_backward_readme_logits(gpu, d, N, ZH):
+    a = make(700 + N + d, ZH[0], ZH[1], N, d, torch.bfloat16, maskfrac=0.2 if N > 65 else 0.0)
+    check_backward(gpu, *a, None, 0.0, 1.0, torch.bfloat16, 2.0 ** -9, f"d={d} N={N} Z,H={ZH}")
 
 
 @pytest.mark.parametrize("d", [32, 64, 128])
