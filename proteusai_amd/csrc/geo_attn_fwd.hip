@@ -70,27 +70,7 @@ __device__ __forceinline__ bool ga_plan_has_wide_tile(const int* __restrict__ wi
     return r;
 }
 
-// The pipelined body over the first half of a doubled grid, the direct-distance body (for workgroups whose
-// queries are spread too widely for the matrix-core distances) over the second; take_all: the pipelined body alone.
-__global__ __launch_bounds__(GA_THREADS, 2)
-void geo_attn_fwd_pipe_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
-                              const uint16_t* __restrict__ V, const float* __restrict__ coords,
-                              const float* __restrict__ sigma, const uint8_t* __restrict__ key_pad,
-                              float* __restrict__ O, float* __restrict__ L,
-                              const int H, const int N, const int ZH, const int n_qtiles, const int n_wgs, const int take_all,
-                              const GaStrides st)
-{
-    extern __shared__ __align__(16) unsigned char ga_dyn_smem[];
-    const int id = (int)blockIdx.x;
-    if (id < n_wgs)
-        geo_attn_fwd_pipe_body(*reinterpret_cast<PipeSmem*>(ga_dyn_smem), id, Q, K, V, coords, sigma, key_pad, O, L,
-                               H, N, ZH, n_qtiles, take_all, st);
-    else
-        geo_attn_fwd_body<true, false, 2>(*reinterpret_cast<Smem*>(ga_dyn_smem), id - n_wgs, Q, K, V, coords, sigma, key_pad, O, L,
-                                          H, N, ZH, n_qtiles, 0, nullptr, 0.f, 1.f, st);
-}
-constexpr size_t GA_PIPE_LDS = sizeof(PipeSmem) > sizeof(Smem) ? sizeof(PipeSmem) : sizeof(Smem);
-static_assert(GA_PIPE_LDS <= 80 * 1024, "two workgroups per compute unit");
+constexpr size_t GA_PIPE_LDS = ga_pipe_lds<64>();
 
 // ---------------- padded batches: a balanced schedule over a persistent grid ----------------
 //
@@ -560,13 +540,13 @@ int launch_attn_pipe(const uint16_t* Q, const uint16_t* K, const uint16_t* V, co
                      const GaStrides& gs, hipStream_t st)
 {
     static std::atomic<unsigned long long> allowed{0ull};
-    const int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel), GA_PIPE_LDS, allowed);
+    const int rc = allow_lds(reinterpret_cast<const void*>(geo_attn_fwd_pipe_kernel<64>), GA_PIPE_LDS, allowed);
     if (rc != (int)hipSuccess) return rc;
     constexpr int BM = GA_WAVES * 64;
     const int n_qtiles = (N + BM - 1) / BM;
     const int ZH = Z * H;
     const unsigned n_wgs = (unsigned)n_qtiles * (unsigned)ZH;
-    hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
+    hipLaunchKernelGGL(geo_attn_fwd_pipe_kernel<64>, dim3(take_all ? n_wgs : 2 * n_wgs), dim3(GA_THREADS), GA_PIPE_LDS, st,
                        Q, K, V, coords, sigma, key_pad_mask, O, L, H, N, ZH, n_qtiles, (int)n_wgs, take_all ? 1 : 0, gs);
     return (int)hipGetLastError();
 }
@@ -656,16 +636,17 @@ int launch_attn_split(const uint16_t* Q, const uint16_t* K, const uint16_t* V, c
     return (int)hipGetLastError();
 }
 
-// d_head and operand type to the kernels.  With two query blocks per wave, d = 64, bf16 operands and the README logits
-// the software-pipelined kernel runs (automatically for large grids of long sequences, or when the tuning asks).
+// d_head and operand type to the kernels.  With two query blocks per wave, d = 64 (here) or 32 (attn_fwd_d32), bf16
+// operands and the README logits the software-pipelined kernel runs (automatically for large grids of long sequences,
+// or when the tuning asks).
 int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint16_t* K, const uint16_t* V, const float* coords,
                 const float* sigma, const uint8_t* key_pad_mask, float* O, float* L, int Z, int H, int N, int tuning,
                 const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st,
                 void* workspace = nullptr, size_t workspace_bytes = 0)
 {
     const bool pipe_tuning = tuning == 5 || tuning == 6 || tuning == 8 || tuning == 9;
-    if (d_head == 32)
-        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,
+    if (d_head == 32)      // (has the pipelined kernel, 5 and 6, but not the schedules over parts)
+        return proteus_internal::attn_fwd_d32(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 8 || tuning == 9) ? 0 : tuning,
                                               beta, min_rbf, max_rbf, gs, st);
     if (d_head == 128)
         return proteus_internal::attn_fwd_d128(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, pipe_tuning ? 0 : tuning,

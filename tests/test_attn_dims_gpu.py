@@ -61,7 +61,9 @@ def check_forward(O, L, Q, K, V, coords, sigma, mask, betas, lo, hi, lse_tol, wh
 @pytest.mark.parametrize("N", [1, 33, 64, 130, 257, 600])
 def test_forward_readme_logits(gpu, d, N):
     Q, K, V, _, coords, sigma, mask = make(500 + N + d, 2, 3, N, d, torch.bfloat16, maskfrac=0.2 if N > 33 else 0.0)
-    for tuning in (0, 1, 2, 3, 4, 7):       # automatic; matrix-core / direct distances; one / two query blocks per wave; keys split
+    # automatic; matrix-core / direct distances; one / two query blocks per wave; keys split; at d = 32 also the
+    # software-pipelined kernel (with and without the direct-distance workgroups beside it)
+    for tuning in (0, 1, 2, 3, 4, 7) + ((5, 6) if d == 32 else ()):
         O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), None if mask is None else mask.to(gpu),
                            return_lse=True, tuning=tuning)
         check_forward(O, L, Q, K, V, coords, sigma, mask, None, 0.0, 1.0, LSE_TOL_BF16, f"d={d} N={N} tuning={tuning}")
@@ -77,9 +79,10 @@ def test_forward_long_ragged_sequence_sampled_rows(gpu, d):
     mask[0, 4700:] = True
     rows = np.sort(np.random.default_rng(d).choice(4700, 48, replace=False))
     betas = torch.tensor([0.6, -0.3])
-    for bt, lo, hi in ((None, 0.0, 1.0), (betas, 0.01, 0.97)):
+    # (tuning 5 at d = 32: the software-pipelined kernel, whose K ring is reused 19 times and whose V ring 26 times)
+    for bt, lo, hi, tuning in ((None, 0.0, 1.0, 0), (betas, 0.01, 0.97, 0)) + (((None, 0.0, 1.0, 5),) if d == 32 else ()):
         O, L = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), return_lse=True,
-                           betas=None if bt is None else bt.to(gpu), min_rbf=lo, max_rbf=hi)
+                           betas=None if bt is None else bt.to(gpu), min_rbf=lo, max_rbf=hi, tuning=tuning)
         O, L = O.cpu().double(), L.cpu().double()
         assert torch.isfinite(O).all() and (O[0, :, 4700:] == 0).all() and torch.isneginf(L[0, :, 4700:]).all()
         if bt is None:
