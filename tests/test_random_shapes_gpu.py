@@ -54,6 +54,10 @@ def test_wavefunction_embeddings(gpu, case):
 def test_attention_forward_and_backward(gpu, case):
     rng = np.random.default_rng(2000 + case)
     Z, H, N = int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.integers(1, 400))
+    if case % 8 == 4:
+        # enough heads for more than 256 backward workgroups of 128 own tokens (both passes together): smaller launches
+        # run workgroups of 64 own tokens at d <= 64, and every other case here is one
+        H = 128 // (Z * ((N + 127) // 128)) + 1
     g = torch.Generator().manual_seed(3000 + case)
     qs = float(rng.choice([0.5, 1.0, 2.0]))
     d = (64, 32, 64, 128)[case % 4]                       # head dimension
@@ -121,7 +125,7 @@ def test_attention_forward_and_backward(gpu, case):
             f"{what} {name}: error / pair mass {(err / pair_mass.clamp_min(1e-300)).max():.3e}"
         if (total.abs() >= 0.25 * pair_mass).all() and total.norm() > 1e-9:
             assert rel_l2(gg.numpy(), total.numpy()) <= 1e-2, f"{what} {name}: {rel_l2(gg.numpy(), total.numpy()):.3e}"
-    if not legacy and d == 64:
+    if not legacy and d in (32, 64):
         # the software-pipelined forward is the default only for large grids: force it on the same inputs
         O5 = pa.geo_attn(Q.to(gpu), K.to(gpu), V.to(gpu), coords.to(gpu), sigma.to(gpu), mask.to(gpu), tuning=5).cpu().double()
         assert torch.isfinite(O5).all(), what
