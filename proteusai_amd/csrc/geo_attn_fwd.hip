@@ -677,13 +677,14 @@ int launch_attn(bool legacy, bool f16, int d_head, const uint16_t* Q, const uint
     }
     if (tuning == 8 || tuning == 9) tuning = 0;
     // The pipelined kernel pays a longer prologue back from about 16 key tiles per workgroup on, and only where its
-    // 256-query workgroups fill the chip twice: measured against the templated body it wins from 512 workgroups and
-    // N = 1024 on (3-11 %), loses below (7-9 % at 256 workgroups of N = 1024, 6-10 % at N = 256 and 512).  A batch that
+    // 256-query workgroups fill most of the chip's 512 slots: measured against the templated body it wins from 416
+    // workgroups and N = 1024 on (3-11 %), loses below (up to 384 workgroups the body's 128-query workgroups are faster,
+    // see launch_attn_dh; 6-10 % at N = 256 and 512).  A batch that
     // comes with a padding mask is taken to be ragged: up to N = 1024 such a batch runs 12-17 % faster on the body's
     // 128-query workgroups (twice as many, half as long: they even out), so it goes there.
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
     const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
-    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
+    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 > 384 && N >= 1024 && !small_ragged)))
         return launch_attn_pipe(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
     return launch_attn_dh<64>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);

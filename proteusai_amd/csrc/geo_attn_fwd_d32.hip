@@ -30,10 +30,10 @@ int proteus_internal::attn_fwd_d32(bool legacy, bool f16, const uint16_t* Q, con
                                    const float* beta, float min_rbf, float max_rbf, const GaStrides& gs, hipStream_t st)
 {
     // tuning 5 / 6: the software-pipelined kernel (6: without the direct-distance workgroups); 0 takes it by the rule of
-    // d = 64 (see launch_attn): from 512 workgroups of 256 queries and N = 1024 on, short ragged batches excepted
+    // d = 64 (see launch_attn): above 384 workgroups of 256 queries, from N = 1024 on, short ragged batches excepted
     const long wgs2 = (long)((N + GA_WAVES * 64 - 1) / (GA_WAVES * 64)) * Z * H;
     const bool small_ragged = key_pad_mask != nullptr && N <= 1024 && wgs2 <= 1024;
-    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 >= 512 && N >= 1024 && !small_ragged)))
+    if (!legacy && (tuning == 5 || tuning == 6 || (tuning == 0 && wgs2 > 384 && N >= 1024 && !small_ragged)))
         return launch_attn_pipe_d32(Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, tuning == 6, gs, st);
     return launch_attn_dh<32>(legacy, f16, Q, K, V, coords, sigma, key_pad_mask, O, L, Z, H, N, (tuning == 5 || tuning == 6) ? 4 : tuning,
                               beta, min_rbf, max_rbf, gs, st);
