@@ -24,6 +24,7 @@
 #include <stdint.h>
 #include <type_traits>
 #include "proteus_hip.h"
+#include "we_ranked.h"
 
 namespace {
 
@@ -60,7 +61,13 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int z    = blockIdx.z;
+    // (observer blocks taken in a rotated order per (y, z), as in the isotropic kernel: in a batch of ragged lengths the
+    // workgroups that are resident together then belong to different parts of their sequences; a padded batch of a
+    // few items is handed out by the number of sources of its items instead, see we_ranked.h)
+    int z = blockIdx.z, ytile = blockIdx.y;
+    const unsigned wa_rot = ((unsigned)(0.6180339887f * (float)gridDim.x + 0.5f)) | 1u;
+    int iblock = (int)((blockIdx.x + wa_rot * (blockIdx.z % gridDim.x) + 5u * blockIdx.y) % gridDim.x);
+    proteus_we::we_ranked_workgroup(mask, N, z, ytile, iblock);
 
     const size_t zN = (size_t)z * (size_t)N;
     const float* az = coordsA + zN * 3;
@@ -68,10 +75,6 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     const uint8_t* mz = mask ? mask + zN : nullptr;
 
     // ---- this lane's observer ----
-    // (observer blocks taken in a rotated order per (y, z), as in the isotropic kernel: in a batch of ragged lengths the
-    // workgroups that are resident together then belong to different parts of their sequences)
-    const unsigned wa_rot = ((unsigned)(0.6180339887f * (float)gridDim.x + 0.5f)) | 1u;
-    const int  iblock = (int)((blockIdx.x + wa_rot * (blockIdx.z % gridDim.x) + 5u * blockIdx.y) % gridDim.x);
     const int  i    = iblock * 64 + lane;
     const bool i_in = i < N;
     const int  ic   = i_in ? i : N - 1;
@@ -82,7 +85,7 @@ void we_aniso_fwd_kernel(const float* __restrict__ coordsA, const float* __restr
     const bool any_valid = __builtin_amdgcn_ballot_w64(i_valid) != 0;   // uniform over the workgroup
 
     // ---- this wave's wavenumbers: kr = k/2pi and ck = cb k/2pi, in revolutions per angstrom ----
-    const int  k0          = SPLIT ? blockIdx.y * KT : (blockIdx.y * WA_WAVES + wave) * KT;
+    const int  k0          = SPLIT ? ytile * KT : (ytile * WA_WAVES + wave) * KT;
     const bool wave_active = k0 < K;
     float kr[KT], ck[KT];
 #pragma unroll

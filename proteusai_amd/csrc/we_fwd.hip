@@ -29,6 +29,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "proteus_hip.h"
+#include "we_ranked.h"
 
 namespace {
 
@@ -283,7 +284,8 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int z    = blockIdx.z;
+    int z      = blockIdx.z;
+    int ytile  = blockIdx.y;
 
     // Workgroup (x, y, z) takes observer block x + a z + 5 y (mod the number of blocks), a = 0.618 of that number made
     // odd: the same set of blocks per (y, z), in another order.  Workgroups that are resident together then belong to
@@ -292,7 +294,10 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     // changes for full ones.
     const unsigned we_rot = ((unsigned)(0.6180339887f * (float)gridDim.x + 0.5f)) | 1u;
     // (32-bit safe: a <= 0.62 x 65536 blocks, z taken modulo the number of blocks first, y < 4096)
-    const int iblock = (int)((blockIdx.x + we_rot * (blockIdx.z % gridDim.x) + 5u * blockIdx.y) % gridDim.x);
+    int iblock = (int)((blockIdx.x + we_rot * (blockIdx.z % gridDim.x) + 5u * blockIdx.y) % gridDim.x);
+
+    // A padded batch of a few items is handed out by the number of sources of its items instead (we_ranked.h)
+    proteus_we::we_ranked_workgroup(mask, N, z, ytile, iblock);
 
     const size_t zN = (size_t)z * (size_t)N;
     const float* cz = coords + zN * 3;
@@ -313,12 +318,12 @@ void we_fwd_kernel(const float* __restrict__ coords, const int layout,
     if (!any_valid) {
         // 64 padded (or out-of-range) observers: zeros, and nothing else to do (in a batch of ragged lengths this is a
         // large share of the workgroups)
-        we_write_zero_rows<KT, SPLIT, MAG>(out, cos_sums, sin_sums, K, zN, i, i_in, wave, blockIdx.y);
+        we_write_zero_rows<KT, SPLIT, MAG>(out, cos_sums, sin_sums, K, zN, i, i_in, wave, ytile);
         return;
     }
 
     // ---- this wave's wavenumbers, converted to revolutions per angstrom ----
-    const int  k0          = SPLIT ? blockIdx.y * KT : (blockIdx.y * WE_WAVES + wave) * KT;
+    const int  k0          = SPLIT ? ytile * KT : (ytile * WE_WAVES + wave) * KT;
     const bool wave_active = k0 < K;
     float kr[KT];
 #pragma unroll

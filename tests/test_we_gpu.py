@@ -330,6 +330,73 @@ def test_cfg4_batch_with_padding(gpu):
     check(got, coords, wn, mask, rows=rows, what="cfg4")
 
 
+@pytest.mark.parametrize("N,d_model,kind", [(640, 64, "ties"), (520, 128, "unaligned"), (1024, 512, "many"), (512, 32, "few tiles")])
+def test_padded_batches_handed_out_by_their_number_of_sources(gpu, N, d_model, kind):
+    # Padded batches of 2 .. 64 items with N >= 512 (up to 4096 workgroups): every workgroup ranks the items by their number
+    # of unpadded sources and takes its place in a list laid over the launch as a snake.  Every (item, observer block,
+    # wavenumber tile) must still be done exactly once: full rows against the oracle, and exact zeros on padded rows
+    # of an output that was filled with NaN.
+    g = torch.Generator().manual_seed(N)
+    if kind == "ties":          # equal counts, an empty item, lengths on and beside the 64-row block borders, a scattered mask
+        lens = [640, 64, 640, 0, 65, 63, 320, 1]
+        Z = len(lens)
+        mask = torch.arange(N)[None, :] >= torch.tensor(lens)[:, None]
+        mask = torch.cat([mask, (torch.rand(1, N, generator=g) < 0.6)], 0)      # fewer sources than its last token says
+        mask[-1, 600] = False
+        Z += 1
+    elif kind == "unaligned":   # rows of the mask that are not multiples of 16 bytes: the byte-wise scan
+        Z = 5
+        lens = torch.randint(1, N + 1, (Z,), generator=g)
+        mask = torch.arange(N)[None, :] >= lens[:, None]
+    elif kind == "many":        # 4 items x 16 blocks x 16 wavenumber tiles: several rows of the snake, the last one partial
+        Z = 4
+        lens = torch.tensor([1024, 130, 777, 512])
+        mask = torch.arange(N)[None, :] >= lens[:, None]
+    else:                       # 64 items, the most that are ranked
+        Z = 64
+        lens = torch.randint(0, N + 1, (Z,), generator=g)
+        mask = torch.arange(N)[None, :] >= lens[:, None]
+    coords, wn = synth.we_inputs(N, seed=N, batch=Z, d_model=d_model)
+    K = wn.numel()
+    for sums in (True, False):
+        c, w, m = coords.to(gpu), wn.to(gpu), mask.to(gpu)
+        got = pa.we_forward(c, w, m, need_sums=sums)
+        out = got[0].cpu().numpy()
+        assert np.isfinite(out).all() and (out[mask.numpy()] == 0).all(), f"{kind} sums={sums}"
+        ref = c_oracle.we(coords.numpy(), wn.numpy(), mask.numpy(), precision="f32")
+        assert rel_l2(out, ref[0]) <= REL_L2_TOL, f"{kind} sums={sums}: {rel_l2(out, ref[0]):.3e}"
+        if sums:
+            for a, r, name in zip(got[1:], ref[1:], ("cos_sums", "sin_sums")):
+                a = a.cpu().numpy()
+                assert (a[mask.numpy()] == 0).all() and rel_l2(a, r) <= REL_L2_TOL, f"{kind} {name}"
+    # the anisotropic kernel takes its workgroups in the same order
+    gb = torch.Generator().manual_seed(N + 1)
+    cb_dir = torch.randn(Z, N, 3, generator=gb)
+    cb_dir = cb_dir / cb_dir.norm(dim=-1, keepdim=True)
+    cb = torch.rand(K, generator=gb) * 4 - 2
+    got = pa.we_aniso_forward(coords.to(gpu), cb_dir.to(gpu), cb.to(gpu), wn.to(gpu), mask.to(gpu))
+    ref = c_oracle.we_aniso(coords.numpy(), cb_dir.numpy(), cb.numpy(), wn.numpy(), mask.numpy())
+    for a, r, name in zip(got, ref, ("out", "d_cb", "d_k")):
+        a = a.cpu().numpy()
+        assert np.isfinite(a).all() and (a[mask.numpy()] == 0).all() and rel_l2(a, r) <= REL_L2_TOL, f"{kind} anisotropic {name}: {rel_l2(a, r):.3e}"
+    # through the raw entry point into buffers full of NaN, every tile width: nothing left unwritten, nothing written twice differently
+    lib = _lib.load()
+    c, w, m = coords.to(gpu).contiguous(), wn.to(gpu), mask.to(gpu).view(torch.uint8).contiguous()
+    base = None
+    for tuning in range(len(_lib.we_variants())):
+        bufs = [torch.full((Z, N, 2 * K), float("nan"), device=gpu), torch.full((Z, N, K), float("nan"), device=gpu),
+                torch.full((Z, N, K), float("nan"), device=gpu)]
+        rc = lib.proteus_we_fwd(c.data_ptr(), 1, w.data_ptr(), m.data_ptr(), bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(),
+                                Z, N, K, tuning, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        o = bufs[0].cpu().numpy()
+        assert all(torch.isfinite(b).all() for b in bufs), f"{kind} variant {tuning}"
+        if base is None:
+            base = o
+        assert rel_l2(o, base) < 1e-5, f"{kind} variant {tuning}"
+
+
 def test_hardware_sincos_and_sqrt_error(gpu):
     # the stated fp32 error of the fast path: v_sin_f32 / v_cos_f32 on revolutions, with and without the
     # explicit range reduction, and r = r2*rsq(r2) with one Newton step (measurement probes: their own library)
