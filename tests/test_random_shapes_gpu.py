@@ -50,6 +50,35 @@ def test_wavefunction_embeddings(gpu, case):
         assert rel_l2(g, r) <= 1e-4, f"{what} aniso {name}: {rel_l2(g, r):.3e}"
 
 
+@pytest.mark.parametrize("case", range(16))
+def test_wavefunction_embeddings_of_padded_batches(gpu, case):
+    # 2 .. 64 items of 512 tokens or more: the launches whose workgroups are handed out by the number of sources of
+    # their items (tail padding, scattered masks, lengths on the block borders and empty items, both together)
+    rng = np.random.default_rng(31000 + case)
+    Z = int(rng.integers(2, 65))
+    N = int(rng.integers(512, max(513, min(1500, 65536 // Z))))
+    K = int(rng.choice([4, 8, 16, 24, 40]))
+    coords = chain(rng, Z, N, 1.0, np.zeros(3))
+    wn = torch.from_numpy(rng.uniform(0.05, 1.5, K).astype(np.float32))
+    kind = case % 4
+    if kind == 0:
+        mask = np.arange(N)[None, :] >= rng.integers(0, N + 1, Z)[:, None]
+    elif kind == 1:
+        mask = rng.random((Z, N)) < rng.uniform(0.1, 0.9, (Z, 1))
+    elif kind == 2:
+        mask = np.arange(N)[None, :] >= rng.choice([N, N // 2, 64, 65, 0], Z)[:, None]
+    else:
+        mask = (np.arange(N)[None, :] >= rng.integers(N // 8, N + 1, Z)[:, None]) | (rng.random((Z, N)) < 0.05)
+    mask = torch.from_numpy(mask)
+    what = f"case {case}: Z={Z} N={N} K={K} kind={kind}"
+    got = pa.we_forward(coords.to(gpu), wn.to(gpu), mask.to(gpu))
+    ref = c_oracle.we(coords.numpy(), wn.numpy(), mask.numpy())
+    for g, r, name in zip(got, ref, ("out", "cos_sums", "sin_sums")):
+        g = g.cpu().numpy()
+        assert np.isfinite(g).all() and (g[mask.numpy()] == 0).all(), f"{what} {name}"
+        assert rel_l2(g, r) <= 1e-4, f"{what} {name}: {rel_l2(g, r):.3e}"
+
+
 @pytest.mark.parametrize("case", range(160))
 def test_attention_forward_and_backward(gpu, case):
     rng = np.random.default_rng(2000 + case)
