@@ -4,6 +4,7 @@ There is no CPU fallback: if the library is missing or a call fails, an
 exception is raised.
 """
 import ctypes
+import functools
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -161,12 +162,27 @@ def geo_attn_variants():
     return [lib.proteus_geo_attn_variant_name(i).decode() for i in range(lib.proteus_geo_attn_num_variants())]
 
 
-def stride_array(*tensors):
-    """(batch, head, token) element strides of [Z,H,N,d] tensors, flattened, as the strided entry points take them."""
-    vals = []
-    for t in tensors:
-        vals += [t.stride(0), t.stride(1), t.stride(2)]
+@functools.lru_cache(maxsize=256)
+def _stride_array_of(vals):
     return (ctypes.c_int64 * len(vals))(*vals)
+
+
+def stride_array(*tensors):
+    """(batch, head, token) element strides of [Z,H,N,d] tensors, flattened, as the strided entry points take them
+    (the arrays are read-only for the library and kept per combination of strides)."""
+    vals = ()
+    for t in tensors:
+        vals += t.stride()[:3]
+    return _stride_array_of(vals)
+
+
+def raw_stream(dev):
+    """Handle of torch's current stream on `dev` for the `stream` argument of the entry points."""
+    import torch
+    try:
+        return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch.cuda.current_device())
+    except AttributeError:       # (a torch without the short cut)
+        return torch.cuda.current_stream(dev).cuda_stream
 
 
 class _NoSwitch:

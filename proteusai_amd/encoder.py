@@ -44,7 +44,7 @@ def add_layer_norm(x, res, norm: nn.LayerNorm):
         rc = lib.proteus_add_layernorm_fwd(xc.data_ptr(), rc_.data_ptr(), None if w is None else w.data_ptr(),
                                            None if b is None else b.data_ptr(), out.data_ptr(), rows, D, float(norm.eps),
                                            _lib.DTYPE_F32 if x.dtype == torch.float32 else _lib.DTYPE_BF16,
-                                           torch.cuda.current_stream(x.device).cuda_stream)
+                                           _lib.raw_stream(x.device))
     _lib.check(rc, "proteus_add_layernorm_fwd")
     return out
 

@@ -6,31 +6,52 @@ Mirrors the reference's Python surface:
 with the logits of README.md:40, s = (q.k/sqrt(d)) * (1 + exp(-|rq-rk|^2/(2 sigma_h^2))),
 plus `geo_attn`, the (Q, K, V, coords, sigma_per_head, key_padding_mask) form.
 """
+import functools
+
 import torch
 import torch.nn as nn
 
 from . import _lib
 
 
+@functools.lru_cache(maxsize=1024)
+def _layout_ok(size, stride, itemsize):
+    per16 = 16 // itemsize
+    return (stride[3] == 1 and stride[2] >= size[3]
+            and all(st >= 0 and st % per16 == 0 for st in stride[:3])
+            and (size[0] == 1 or stride[0] > 0) and (size[1] == 1 or stride[1] > 0)
+            and size[2] * stride[2] * itemsize < 2 ** 31)
+
+
 def _rows_ok(t, itemsize):
     """Can the kernels read / write this [Z,H,N,d] tensor in place?  Rows of d contiguous elements, 16-byte
     aligned, no negative or overlapping-row strides; the batch, head and token strides are otherwise free."""
-    if t.is_contiguous():
-        return t.data_ptr() % 16 == 0
-    per16 = 16 // itemsize
-    return (t.stride(3) == 1 and t.data_ptr() % 16 == 0 and t.stride(2) >= t.size(3)
-            and all(st >= 0 and st % per16 == 0 for st in t.stride()[:3])
-            and (t.size(0) == 1 or t.stride(0) > 0) and (t.size(1) == 1 or t.stride(1) > 0)
-            and t.size(2) * t.stride(2) * itemsize < 2 ** 31)
+    if t.data_ptr() % 16 != 0:
+        return False
+    return t.is_contiguous() or _layout_ok(tuple(t.shape), t.stride(), itemsize)
 
 
 def _operand(t, dtype=torch.bfloat16):
     """16-bit view of an operand the kernels can read where it lies (a copy only if it has to be cast or its rows
     are not contiguous)."""
-    t = t.detach()
+    if t.requires_grad:
+        t = t.detach()
     if t.dtype != dtype:
         t = t.to(dtype)
     return t if _rows_ok(t, 2) else t.contiguous()
+
+
+def _f32(t, dev):
+    """fp32, contiguous, on `dev`, outside autograd: the tensor itself where it already is all that."""
+    if t.dtype == torch.float32 and t.device == dev and not t.requires_grad and t.is_contiguous():
+        return t
+    return t.detach().to(device=dev, dtype=torch.float32).contiguous()
+
+
+def _mask_bytes(mask, dev):
+    if mask.dtype == torch.bool and mask.device == dev and mask.is_contiguous():
+        return mask.view(torch.uint8)
+    return mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
 
 
 def _operand_type(operand_dtype, legacy):
@@ -87,13 +108,13 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     legacy = betas is not None
     op_dtype, op_type = _operand_type(operand_dtype, legacy)
     q, k, v = _operand(Q, op_dtype), _operand(K, op_dtype), _operand(V, op_dtype)
-    c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
-    s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
+    c = _f32(coords, dev)
+    s = _f32(sigma, dev)
     m = None
     if key_padding_mask is not None:
         if tuple(key_padding_mask.shape) != (Z, N):
             raise AssertionError(f"mask must be of shape ({Z}, {N}), not {tuple(key_padding_mask.shape)}")
-        m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
+        m = _mask_bytes(key_padding_mask, dev)
     if token_major_out:
         O = torch.empty(Z, N, H, d, dtype=torch.float32, device=dev).permute(0, 2, 1, 3)
     else:
@@ -102,7 +123,7 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
     if Z == 0 or H == 0 or N == 0:
         return (O, L) if return_lse else O
     with _lib.on_device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.raw_stream(dev)
         ws_bytes = lib.proteus_geo_attn_fwd_workspace_bytes(Z, H, N, d, int(tuning)) if not legacy else 0
         if ws_bytes:
             # long sequences: with a workspace the library may cut the key loop of a (batch, head, query tile) item into
@@ -125,7 +146,7 @@ def geo_attn(Q, K, V, coords, sigma, key_padding_mask=None, return_lse: bool = F
         else:
             if betas.dim() != 1 or betas.size(0) != H:
                 raise AssertionError(f"number of betas must be equal to nheads, not {tuple(betas.shape)} and {H=}")
-            bt = betas.detach().to(device=dev, dtype=torch.float32).contiguous()
+            bt = _f32(betas, dev)
             if _is_plain(q, k, v, O):
                 rc = lib.proteus_geo_attn_legacy_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), c.data_ptr(), s.data_ptr(),
                                                      bt.data_ptr(), None if m is None else m.data_ptr(),
@@ -159,7 +180,7 @@ def _delta(O, dO):
     strides = None if (O.is_contiguous() and dO.is_contiguous()) else _lib.stride_array(O, dO)
     with _lib.on_device(O.device):
         rc = _lib.load().proteus_geo_attn_delta(O.data_ptr(), dO.data_ptr(), strides, D.data_ptr(), Z, H, N, d,
-                                                _DELTA_DTYPES[dO.dtype], torch.cuda.current_stream(O.device).cuda_stream)
+                                                _DELTA_DTYPES[dO.dtype], _lib.raw_stream(O.device))
     _lib.check(rc, "proteus_geo_attn_delta")
     return D
 
@@ -183,13 +204,11 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     q, k, v = _operand(Q, op_dtype), _operand(K, op_dtype), _operand(V, op_dtype)
     D = _delta(O.detach(), dO.detach())
     do = _operand(dO, op_dtype)
-    c = coords.detach().to(device=dev, dtype=torch.float32).contiguous()
-    s = sigma.detach().to(device=dev, dtype=torch.float32).contiguous()
-    lse = L.detach().to(torch.float32).contiguous()
-    m = None
-    if key_padding_mask is not None:
-        m = key_padding_mask.to(device=dev, dtype=torch.bool).contiguous().view(torch.uint8)
-    bt = None if betas is None else betas.detach().to(device=dev, dtype=torch.float32).contiguous()
+    c = _f32(coords, dev)
+    s = _f32(sigma, dev)
+    lse = _f32(L, dev)
+    m = None if key_padding_mask is None else _mask_bytes(key_padding_mask, dev)
+    bt = None if betas is None else _f32(betas, dev)
     # gradients in the memory order of their operands (dense), so that what consumes them needs no reshuffle
     def like(t):
         g = torch.empty_like(t, dtype=torch.float32)
@@ -206,7 +225,7 @@ def geo_attn_backward(Q, K, V, O, L, dO, coords, sigma, key_padding_mask=None, b
     if Z == 0 or H == 0 or N == 0:
         return dQ, dK, dV, d_sigma, d_beta
     with _lib.on_device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.raw_stream(dev)
         tail = (c.data_ptr(), s.data_ptr(), None if bt is None else bt.data_ptr(), None if m is None else m.data_ptr(),
                 lse.data_ptr(), D.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
                 d_sigma.data_ptr(), None if d_beta is None else d_beta.data_ptr(),
@@ -295,6 +314,12 @@ def geometric_attn_qkv(qkv, coords, spreads, betas=None, mask=None, min_rbf=0.00
         raise AssertionError(f"qkv must be of shape (batch, N, 3, heads, d_k), not {tuple(qkv.shape)}")
     if not _rows_ok(qkv[:, :, 0].permute(0, 2, 1, 3), qkv.element_size()):
         qkv = qkv.contiguous()
+    if not (torch.is_grad_enabled() and (qkv.requires_grad or spreads.requires_grad or (betas is not None and betas.requires_grad))):
+        # nothing to differentiate: the forward alone, without an autograd node
+        Q, K, V = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        O = geo_attn(Q, K, V, coords, spreads, mask, betas=betas, min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_spreads,
+                     token_major_out=True, operand_dtype=operand_dtype)
+        return O if out_dtype is None or out_dtype == O.dtype else O.to(out_dtype)
     return _geometric_attn_qkv.apply(qkv, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads, out_dtype, operand_dtype)
 
 
@@ -312,6 +337,11 @@ def geometric_attn(Q, K, V, coords, spreads, betas=None, mask=None, min_rbf=0.00
     """
     if betas is None and (min_rbf > 0.0 or max_rbf < 1.0):
         raise NotImplementedError("the [min_rbf, max_rbf] pair mask belongs to the beta-weighted logits; pass betas")
+    if not (torch.is_grad_enabled() and (Q.requires_grad or K.requires_grad or V.requires_grad or spreads.requires_grad
+                                         or (betas is not None and betas.requires_grad))):
+        O = geo_attn(Q, K, V, coords, spreads, mask, betas=betas, min_rbf=min_rbf, max_rbf=max_rbf, check_sigma=check_spreads,
+                     token_major_out=token_major_out, operand_dtype=operand_dtype)
+        return O if out_dtype is None or out_dtype == O.dtype else O.to(out_dtype)
     return _geometric_attn.apply(Q, K, V, coords, spreads, betas, mask, min_rbf, max_rbf, check_spreads,
                                  token_major_out, out_dtype, operand_dtype)
 

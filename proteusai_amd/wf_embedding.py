@@ -59,7 +59,7 @@ def we_forward(coords, wavenumbers, mask=None, tuning: int = 0, magnitude_type: 
     if Z == 0 or N == 0 or K == 0:
         return out, cos_sums, sin_sums
     with _lib.on_device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.raw_stream(dev)
         if dropout_p != 0.0:
             if rng_seed is None:
                 rng_seed = int(torch.randint(0, 2 ** 32, (1,), dtype=torch.int64).item())
@@ -89,7 +89,7 @@ def _bwd_prepare(dO, *saved):
     ts = [dO.contiguous().float()] + [None if t is None else t.contiguous().float() for t in saved]
     lib = _lib.load()
     ws = torch.empty(max(1, lib.proteus_we_bwd_workspace_bytes(Z, N, K2 // 2) // 4), dtype=torch.float32, device=dO.device)
-    return lib, ts, ws, Z, N, K2 // 2, torch.cuda.current_stream(dO.device).cuda_stream
+    return lib, ts, ws, Z, N, K2 // 2, _lib.raw_stream(dO.device)
 
 
 def we_backward(dO, cos_sums, sin_sums):
@@ -202,7 +202,7 @@ def we_aniso_forward(coordsA, coordsB, cb_magnitudes, wavenumbers, mask=None, tu
     if Z == 0 or N == 0 or K == 0:
         return out, d_cb, d_k
     with _lib.on_device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.raw_stream(dev)
         rc = lib.proteus_we_aniso_fwd(a.data_ptr(), b.data_ptr(), _lib.COORDS_AOS, cb.data_ptr(), w.data_ptr(),
                                       None if m is None else m.data_ptr(),
                                       out.data_ptr(), d_cb.data_ptr() if partials else None, d_k.data_ptr() if partials else None,
