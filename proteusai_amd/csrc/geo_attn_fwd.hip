@@ -430,16 +430,13 @@ void geo_attn_fwd_split_kernel(const uint16_t* __restrict__ Q, const uint16_t* _
     // first workgroup before any gets its second).  The second half takes the parts in reverse, so the longest part is
     // paired with the shortest (or with none): when the short one is done the long one has the unit to itself.
     // The heads keep their pairing (a head of small sigma with one of large sigma, see below).
-#ifndef GB_SPLIT_MIRROR
-#define GB_SPLIT_MIRROR 1
-#endif
     // (Only where the parts differ in length: with equal parts, a single sequence, the order of the query tiles is worth
     // more.  cfg 4 x 8 x 4096 padded 146 -> 141 us, 8 x 8 x 2048 padded 109 -> 101, 2 x 8 x 8192 padded 125 -> 119; one
     // sequence of 8192 tokens would lose 2 %.)
     int p = (int)blockIdx.x;
     auto part_len = [&](const int r) { const int c = (bs.n_eff[order[r]] + GA_BN - 1) / GA_BN; return (c + splits[r] - 1) / splits[r]; };
     const bool uneven = part_len(0) != part_len(Z - 1);
-    const bool mirrored = GB_SPLIT_MIRROR && uneven && p >= (cap >> 1) && p < cap;
+    const bool mirrored = uneven && p >= (cap >> 1) && p < cap;
     if (mirrored) p = cap - 1 - (p - (cap >> 1));
     if (p < n_parts) {
         int r = 0;
